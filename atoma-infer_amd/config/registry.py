@@ -50,10 +50,11 @@ def resolve_architecture(obj: Dict[str, Any], where: str = "config.json") -> Arc
         names += [a for a in archs if isinstance(a, str)]
     elif isinstance(archs, str):
         names.append(archs)
-    if isinstance(obj.get("model_type"), str):
-        names.append(obj["model_type"])
+    for k in ("architecture", "model_type"):
+        if isinstance(obj.get(k), str):
+            names.append(obj[k])
     if not names:
-        raise ConfigError(f"{where}: neither 'architectures' nor 'model_type' names the model; "
+        raise ConfigError(f"{where}: neither 'architectures', 'architecture' nor 'model_type' names the model; "
                           f"known architectures: {', '.join(known_architectures())}")
     for n in names:
         if n in _ARCHITECTURES:

@@ -11,6 +11,9 @@
 // h / (nh / nkv) (csrc/kernels/flash_fwd_kernel.h:593).  With slopes (one per query head) the score of key j for the
 // token at p gains slopes[h] * (j - p), a bias that is linear in the distance (the reference's kernels take such
 // slopes too: csrc/kernels/mask.h:155-157, 179-186; its Llama passes none).
+// With chunk > 0 the token at p sees only the keys of its own chunk of positions, [(p / chunk) * chunk, p]
+// (chunks count from position 0 of the request).  With sinks (one float32 per query head) the softmax denominator
+// also holds exp(sinks[h]): a weight that belongs to no key and carries no value.
 #include "common.h"
 #include "cache_layout.h"
 
@@ -25,7 +28,7 @@ paged_attention_generic_kernel(const TQ* __restrict__ q, int q_stride, const TC*
                                const int32_t* __restrict__ block_tables, int max_blocks,
                                const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
                                float scale, int window, int page_size, int nh, int nkv, int hd,
-                               const float* __restrict__ slopes) {
+                               const float* __restrict__ slopes, int chunk, const float* __restrict__ sinks) {
   __shared__ float qs[kMaxHead];
   __shared__ float ps[kWave];
   __shared__ int32_t pg[kWave];
@@ -35,7 +38,8 @@ paged_attention_generic_kernel(const TQ* __restrict__ q, int q_stride, const TC*
   const int s = token_seq[t], p = positions[t];
   const int kvh = h / (nh / nkv);
   const int32_t* table = block_tables + (size_t)s * max_blocks;
-  const int first = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  int first = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  if (chunk > 0 && (p / chunk) * chunk > first) first = (p / chunk) * chunk;
   const float slope = slopes ? slopes[h] : 0.f;
 
   for (int d = lane; d < hd; d += kWave) qs[d] = to_f32(q[(size_t)t * q_stride + (size_t)h * hd + d]);
@@ -85,6 +89,15 @@ paged_attention_generic_kernel(const TQ* __restrict__ q, int q_stride, const TC*
       }
     }
   }
+  if (sinks) {
+    // the sink joins the denominator under the common maximum
+    const float sk = sinks[h];
+    const float m_new = fmaxf(m, sk);
+    const float corr = expf(m - m_new);
+    l = l * corr + expf(sk - m_new);
+#pragma unroll
+    for (int i = 0; i < kMaxHead / kWave; ++i) acc[i] *= corr;
+  }
   const float inv = 1.0f / l;  // at least the token's own key is visible, so l > 0
 #pragma unroll
   for (int i = 0; i < kMaxHead / kWave; ++i) {
@@ -98,7 +111,7 @@ extern "C" int atoma_paged_attention_generic(const void* q, int q_stride, const 
                                              const int32_t* block_tables, int max_blocks, const int32_t* token_seq,
                                              const int32_t* positions, float scale, int window, int page_size,
                                              int n_tokens, int nh, int nkv, int hd, const float* slopes,
-                                             hipStream_t stream) {
+                                             int chunk, const float* sinks, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (hd <= 0 || hd > kMaxHead || nkv <= 0 || nh % nkv || page_size <= 0 || max_blocks <= 0 || nh > 65535)
     return ATOMA_ERR_SHAPE;
@@ -106,7 +119,7 @@ extern "C" int atoma_paged_attention_generic(const void* q, int q_stride, const 
 #define ATOMA_ATTN(TQ, TC)                                                                                       \
   hipLaunchKernelGGL((paged_attention_generic_kernel<TQ, TC>), grid, block, 0, stream, (const TQ*)q, q_stride, \
                      (const TC*)kcache, (const TC*)vcache, (TQ*)out, out_stride, block_tables, max_blocks,      \
-                     token_seq, positions, scale, window, page_size, nh, nkv, hd, slopes)
+                     token_seq, positions, scale, window, page_size, nh, nkv, hd, slopes, chunk, sinks)
   if (act_dtype == kF32 && cache_dtype == kF32) ATOMA_ATTN(float, float);
   else if (act_dtype == kBF16 && cache_dtype == kBF16) ATOMA_ATTN(bf16_t, bf16_t);
   else if (act_dtype == kF32 && cache_dtype == kBF16) ATOMA_ATTN(float, bf16_t);

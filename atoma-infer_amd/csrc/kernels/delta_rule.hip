@@ -1,0 +1,251 @@
+// The gated delta rule: a recurrent mixer whose state is one float32 matrix S [dim, vdim] per head and request.
+//
+// Per token and head (q, k of size dim, unit length; v of size vdim; beta a scalar; g a decay per key channel):
+//   S <- diag(g) S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q          (the read-out sees the token's write)
+// Everything here is float32.  Four kernels:
+//   delta_prepare      per token: short causal convolution over time and SiLU of the q, k, v projections (the taps - 1
+//                      inputs before an entry's first token come from the request's state), q and k to unit length per
+//                      head (q also times dim^-1/2), beta = sigmoid(b), g = exp(-exp(A_log) softplus(a + dt_bias));
+//   delta_conv_state   per request: the last taps - 1 inputs of the convolution, for the request's next step;
+//   delta_scan         per (request, head, 8 columns of S): the recurrence over the entry's tokens in order, S read from
+//                      the request's state slot before and written back after.  A column of S lives in the registers
+//                      of 8 neighbouring lanes (dim / 8 rows each, rounded up), so a token costs a lane a few dozen
+//                      multiply-adds and one three-step exchange among those lanes;
+//   delta_out          per token and head: o / sqrt(mean(o^2) + eps) * w * sigmoid(gate), in the activation dtype.
+// The order of every sum depends on the sizes alone, so a token's result does not depend on how the request was cut
+// into steps or on what else the step holds.
+//
+// State of a request (float32, one row of the state tensor):  [taps - 1][conv channels]  then  [heads][vdim][dim].
+#include "common.h"
+
+using namespace atoma;
+
+struct DeltaShape {
+  int heads, kv_heads, dim, vdim, taps;
+  int ldp;                 // row stride of the projections
+  int off_q, off_k, off_v, off_b;   // first columns of the q, k, v and b projections in a row
+};
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float softplusf_(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+// conv channels: q (kv_heads * dim), then k (the same), then v (heads * vdim); taps_w [channels, taps] in that order
+__global__ void __launch_bounds__(256)
+delta_prepare_kernel(const float* __restrict__ proj, DeltaShape sh, const int32_t* __restrict__ token_seq,
+                     const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
+                     const float* __restrict__ state, size_t state_stride, const float* __restrict__ taps_w,
+                     const float* __restrict__ dt_pre, const float* __restrict__ dt_bias,
+                     const float* __restrict__ a_log, float* __restrict__ qn, float* __restrict__ kn,
+                     float* __restrict__ vn, float* __restrict__ beta, float* __restrict__ decay) {
+  extern __shared__ float act[];       // the token's channels after convolution and SiLU
+  const int t = blockIdx.x;
+  const int e = token_seq[t];
+  const int n = t - q_start[e];        // the token's index inside its entry
+  const int nqk = sh.kv_heads * sh.dim, nv = sh.heads * sh.vdim, channels = 2 * nqk + nv;
+  const float* conv_state = state + (size_t)state_slots[e] * state_stride;
+  for (int c = threadIdx.x; c < channels; c += 256) {
+    const int col = c < nqk ? sh.off_q + c : c < 2 * nqk ? sh.off_k + (c - nqk) : sh.off_v + (c - 2 * nqk);
+    float y = 0.f;
+    for (int j = 0; j < sh.taps; ++j) {
+      const int s = n - (sh.taps - 1) + j;      // index inside the entry of the input under tap j
+      const float x = s >= 0 ? proj[(size_t)(t - (sh.taps - 1) + j) * sh.ldp + col]
+                             : conv_state[(size_t)(sh.taps - 1 + s) * channels + c];
+      y = fmaf(taps_w[(size_t)c * sh.taps + j], x, y);
+    }
+    act[c] = y * sigmoidf_(y);
+  }
+  __syncthreads();
+  // unit length per head: a wave a head
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float q_scale = 1.0f / sqrtf((float)sh.dim);
+  for (int hh = wave; hh < 2 * sh.kv_heads; hh += 4) {
+    const float* x = act + (size_t)hh * sh.dim;
+    float ss = 0.f;
+    for (int i = lane; i < sh.dim; i += 64) ss += x[i] * x[i];
+    ss = wave_sum(ss);
+    const bool is_q = hh < sh.kv_heads;
+    const float inv = (is_q ? q_scale : 1.0f) / sqrtf(ss + 1e-6f);
+    float* dst = (is_q ? qn : kn) + (size_t)t * nqk + (size_t)(is_q ? hh : hh - sh.kv_heads) * sh.dim;
+    for (int i = lane; i < sh.dim; i += 64) dst[i] = x[i] * inv;
+  }
+  for (int c = threadIdx.x; c < nv; c += 256) vn[(size_t)t * nv + c] = act[2 * nqk + c];
+  for (int h = threadIdx.x; h < sh.heads; h += 256)
+    beta[(size_t)t * sh.heads + h] = sigmoidf_(proj[(size_t)t * sh.ldp + sh.off_b + h]);
+  const int nd = sh.heads * sh.dim;
+  for (int c = threadIdx.x; c < nd; c += 256) {
+    const float rate = expf(a_log[c / sh.dim]);
+    decay[(size_t)t * nd + c] = expf(-rate * softplusf_(dt_pre[(size_t)t * nd + c] + dt_bias[c]));
+  }
+}
+
+// one thread a (entry, channel): the state's rows in ascending order, so that a row is read before it is overwritten
+__global__ void __launch_bounds__(256)
+delta_conv_state_kernel(const float* __restrict__ proj, DeltaShape sh, const int32_t* __restrict__ q_start,
+                        const int32_t* __restrict__ state_slots, float* __restrict__ state, size_t state_stride) {
+  const int e = blockIdx.y;
+  const int nqk = sh.kv_heads * sh.dim, nv = sh.heads * sh.vdim, channels = 2 * nqk + nv;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= channels) return;
+  const int first = q_start[e], count = q_start[e + 1] - first;
+  const int col = c < nqk ? sh.off_q + c : c < 2 * nqk ? sh.off_k + (c - nqk) : sh.off_v + (c - 2 * nqk);
+  float* st = state + (size_t)state_slots[e] * state_stride;
+  const int keep = sh.taps - 1;
+  for (int r = 0; r < keep; ++r) {
+    const int s = count - keep + r;     // index inside the entry of the input that row r holds afterwards
+    st[(size_t)r * channels + c] = s >= 0 ? proj[(size_t)(first + s) * sh.ldp + col] : st[(size_t)(r + count) * channels + c];
+  }
+}
+
+// R: rows of S a lane holds; 8 lanes share a column, so dim <= 8 R
+template <int R>
+__global__ void __launch_bounds__(64)
+delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vn,
+                  const float* __restrict__ beta, const float* __restrict__ decay, DeltaShape sh,
+                  const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
+                  float* __restrict__ state, size_t state_stride, size_t s_offset, float* __restrict__ o) {
+  const int lane = threadIdx.x;
+  const int col = blockIdx.x * 8 + (lane >> 3), part = lane & 7;
+  const int h = blockIdx.y, e = blockIdx.z;
+  const int kv = h / (sh.heads / sh.kv_heads);
+  const int dim = sh.dim, vdim = sh.vdim;
+  const bool col_ok = col < vdim;
+  const int i0 = part * R;
+  const int first = q_start[e], count = q_start[e + 1] - first;
+  float* sp = state + (size_t)state_slots[e] * state_stride + s_offset +
+              ((size_t)h * vdim + (col_ok ? col : 0)) * dim + i0;
+  float s[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) s[r] = (col_ok && i0 + r < dim) ? sp[r] : 0.f;
+
+  const int nqk = sh.kv_heads * dim, nd = sh.heads * dim, nv = sh.heads * vdim;
+  struct Tok {
+    float q[R], k[R], g[R], v, b;
+  };
+  auto load = [&](Tok& x, int n) {
+    const size_t t = (size_t)(first + n);
+    const float* qp = qn + t * nqk + (size_t)kv * dim + i0;
+    const float* kp = kn + t * nqk + (size_t)kv * dim + i0;
+    const float* gp = decay + t * nd + (size_t)h * dim + i0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const bool ok = i0 + r < dim;
+      x.q[r] = ok ? qp[r] : 0.f;
+      x.k[r] = ok ? kp[r] : 0.f;
+      x.g[r] = ok ? gp[r] : 0.f;
+    }
+    x.v = col_ok ? vn[t * nv + (size_t)h * vdim + col] : 0.f;
+    x.b = beta[t * sh.heads + h];
+  };
+  Tok cur, nxt;
+  if (count > 0) load(cur, 0);
+  for (int n = 0; n < count; ++n) {
+    if (n + 1 < count) load(nxt, n + 1);
+    float d1 = 0.f, d2 = 0.f, kq = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      s[r] *= cur.g[r];
+      d1 = fmaf(s[r], cur.k[r], d1);
+      d2 = fmaf(s[r], cur.q[r], d2);
+      kq = fmaf(cur.k[r], cur.q[r], kq);
+    }
+#pragma unroll
+    for (int off = 1; off < 8; off <<= 1) {
+      d1 += __shfl_xor(d1, off, 64);
+      d2 += __shfl_xor(d2, off, 64);
+      kq += __shfl_xor(kq, off, 64);
+    }
+    const float u = cur.b * (cur.v - d1);
+    // o = S_new^T q with S_new = diag(g) S + k u^T
+    if (part == 0 && col_ok) o[(size_t)(first + n) * nv + (size_t)h * vdim + col] = fmaf(u, kq, d2);
+#pragma unroll
+    for (int r = 0; r < R; ++r) s[r] = fmaf(cur.k[r], u, s[r]);
+    cur = nxt;
+  }
+  if (col_ok) {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (i0 + r < dim) sp[r] = s[r];
+  }
+}
+
+template <typename TO>
+__global__ void __launch_bounds__(256)
+delta_out_kernel(const float* __restrict__ o, const float* __restrict__ gate_pre, const float* __restrict__ w,
+                 float eps, TO* __restrict__ out, int heads, int vdim) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int h = wave; h < heads; h += 4) {
+    const size_t base = ((size_t)t * heads + h) * vdim;
+    float ss = 0.f;
+    for (int j = lane; j < vdim; j += 64) ss += o[base + j] * o[base + j];
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
+    for (int j = lane; j < vdim; j += 64)
+      out[base + j] = from_f32<TO>(o[base + j] * inv * w[j] * sigmoidf_(gate_pre[base + j]));
+  }
+}
+
+static bool shape_ok(const DeltaShape& sh) {
+  return sh.heads > 0 && sh.kv_heads > 0 && sh.heads % sh.kv_heads == 0 && sh.dim > 0 && sh.dim <= 256 && sh.vdim > 0 &&
+         sh.taps >= 1 && sh.taps <= 64 && sh.ldp > 0;
+}
+
+extern "C" int atoma_delta_prepare(const float* proj, int ldp, int off_q, int off_k, int off_v, int off_b, int heads,
+                                   int kv_heads, int dim, int vdim, int taps, const int32_t* token_seq,
+                                   const int32_t* q_start, const int32_t* state_slots, float* state,
+                                   size_t state_stride, const float* taps_w, const float* dt_pre, const float* dt_bias,
+                                   const float* a_log, float* qn, float* kn, float* vn, float* beta, float* decay,
+                                   int n_tokens, int n_entries, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  DeltaShape sh{heads, kv_heads, dim, vdim, taps, ldp, off_q, off_k, off_v, off_b};
+  if (!shape_ok(sh) || n_entries <= 0 || n_entries > 65535) return ATOMA_ERR_SHAPE;
+  const int channels = 2 * kv_heads * dim + heads * vdim;
+  if ((size_t)channels * sizeof(float) > 60 * 1024) return ATOMA_ERR_SHAPE;
+  hipLaunchKernelGGL(delta_prepare_kernel, dim3(n_tokens), dim3(256), channels * sizeof(float), stream, proj, sh,
+                     token_seq, q_start, state_slots, state, state_stride, taps_w, dt_pre, dt_bias, a_log, qn, kn, vn,
+                     beta, decay);
+  ATOMA_LAUNCH_CHECK();
+  if (taps > 1) {
+    hipLaunchKernelGGL(delta_conv_state_kernel, dim3((channels + 255) / 256, n_entries), dim3(256), 0, stream, proj, sh,
+                       q_start, state_slots, state, state_stride);
+    ATOMA_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+extern "C" int atoma_delta_scan(const float* qn, const float* kn, const float* vn, const float* beta,
+                                const float* decay, int heads, int kv_heads, int dim, int vdim, int taps,
+                                const int32_t* q_start, const int32_t* state_slots, float* state, size_t state_stride,
+                                int n_entries, float* o, hipStream_t stream) {
+  if (n_entries <= 0) return 0;
+  DeltaShape sh{heads, kv_heads, dim, vdim, taps, 1, 0, 0, 0, 0};
+  if (!shape_ok(sh) || n_entries > 65535 || heads > 65535) return ATOMA_ERR_SHAPE;
+  const size_t s_offset = (size_t)(taps - 1) * (2 * kv_heads * dim + heads * vdim);
+  dim3 grid((vdim + 7) / 8, heads, n_entries), block(64);
+#define ATOMA_SCAN(R_)                                                                                            \
+  hipLaunchKernelGGL((delta_scan_kernel<R_>), grid, block, 0, stream, qn, kn, vn, beta, decay, sh, q_start,       \
+                     state_slots, state, state_stride, s_offset, o)
+  if (dim <= 16) ATOMA_SCAN(2);
+  else if (dim <= 32) ATOMA_SCAN(4);
+  else if (dim <= 64) ATOMA_SCAN(8);
+  else if (dim <= 128) ATOMA_SCAN(16);
+  else ATOMA_SCAN(32);
+#undef ATOMA_SCAN
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int atoma_delta_out(const float* o, const float* gate_pre, const float* w, float eps, void* out,
+                               int out_dtype, int n_tokens, int heads, int vdim, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (heads <= 0 || vdim <= 0) return ATOMA_ERR_SHAPE;
+  if (out_dtype == kF32)
+    hipLaunchKernelGGL((delta_out_kernel<float>), dim3(n_tokens), dim3(256), 0, stream, o, gate_pre, w, eps,
+                       (float*)out, heads, vdim);
+  else if (out_dtype == kBF16)
+    hipLaunchKernelGGL((delta_out_kernel<bf16_t>), dim3(n_tokens), dim3(256), 0, stream, o, gate_pre, w, eps,
+                       (bf16_t*)out, heads, vdim);
+  else
+    return ATOMA_ERR_DTYPE;
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}

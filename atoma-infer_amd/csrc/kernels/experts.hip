@@ -1,0 +1,189 @@
+// Feed-forward layers that route every token to a few of many experts.
+//
+//   route_topk    per token: scores = sigmoid(router logits) in float32, the `top` largest (the lower index wins a
+//                 tie) with their scores: a (token, choice) pair is a "slot", numbered token * top + choice;
+//   route_group   one workgroup: slots ordered by expert (perm), where each expert's slots start (offsets), and the
+//                 list of row tiles (expert, first place in perm) that the products below walk.  Which place a slot
+//                 gets inside its expert's range is not fixed; no result depends on it, since every row of a product
+//                 is computed by itself;
+//   expert_gemm   C[row(slot)] = (scale[slot] * A[src(slot)]) . W[expert]^T for all slots, tile by tile: true float32
+//                 multiply-adds over float32 or bfloat16 operands, K in ascending order, so a row's result does not
+//                 depend on the batch around it.  src is the slot's token (first product: the token's input, times its
+//                 score) or the slot itself (second product); the second product writes choice c of token t to row
+//                 c * T + t, so that the choices of a token lie in planes which the next norm adds in order.
+#include "common.h"
+
+using namespace atoma;
+
+constexpr int kTileM = 64, kTileN = 64, kStepK = 16;
+
+__global__ void __launch_bounds__(256)
+route_topk_kernel(const float* __restrict__ logits, int ld, int experts, int top, int32_t* __restrict__ ids,
+                  float* __restrict__ weights, int n_tokens) {
+  // a wave a token; lane l holds experts l, l + 64, ...
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= n_tokens) return;
+  constexpr int PER = 16;      // experts <= 1024
+  float sc[PER];
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int e = lane + j * 64;
+    sc[j] = e < experts ? 1.0f / (1.0f + expf(-logits[(size_t)t * ld + e])) : -1.f;
+  }
+  for (int c = 0; c < top; ++c) {
+    float best = -2.f;
+    int arg = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+      if (sc[j] > best) best = sc[j], arg = lane + j * 64;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, 64);
+      const int oa = __shfl_xor(arg, off, 64);
+      if (ob > best || (ob == best && oa < arg)) best = ob, arg = oa;
+    }
+    if (arg >= experts) arg = c;     // logits that are no numbers: still an expert of the layer
+    if (lane == 0) {
+      ids[(size_t)t * top + c] = arg;
+      weights[(size_t)t * top + c] = best;
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+      if (lane + j * 64 == arg) sc[j] = -1.f;
+  }
+}
+
+__global__ void __launch_bounds__(1024)
+route_group_kernel(const int32_t* __restrict__ ids, int n_slots, int experts, int32_t* __restrict__ perm,
+                   int32_t* __restrict__ offsets, int32_t* __restrict__ tiles, int max_tiles) {
+  __shared__ int32_t counts[1024];
+  __shared__ int32_t cursor[1024];
+  for (int e = threadIdx.x; e < experts; e += 1024) counts[e] = 0;
+  __syncthreads();
+  for (int s = threadIdx.x; s < n_slots; s += 1024) atomicAdd(&counts[ids[s]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, n = 0;
+    for (int e = 0; e < experts; ++e) {
+      offsets[e] = at;
+      cursor[e] = at;
+      for (int r = 0; r < counts[e]; r += kTileM) {
+        tiles[2 * n] = e;
+        tiles[2 * n + 1] = at + r;
+        ++n;
+      }
+      at += counts[e];
+    }
+    offsets[experts] = at;
+    for (; n < max_tiles; ++n) tiles[2 * n] = -1, tiles[2 * n + 1] = 0;
+  }
+  __syncthreads();
+  for (int s = threadIdx.x; s < n_slots; s += 1024) perm[atomicAdd(&cursor[ids[s]], 1)] = s;
+}
+
+template <typename TA, typename TW, typename TC>
+__global__ void __launch_bounds__(256)
+expert_gemm_kernel(const TA* __restrict__ a, int lda, int a_div, const float* __restrict__ scale,
+                   const TW* __restrict__ w, TC* __restrict__ c, int ldc, int N, int K,
+                   const int32_t* __restrict__ perm, const int32_t* __restrict__ offsets,
+                   const int32_t* __restrict__ tiles, int top, int plane_rows) {
+  __shared__ float as[kStepK][kTileM + 4];
+  __shared__ float ws[kStepK][kTileN + 4];
+  __shared__ int32_t slot_of[kTileM];
+  const int e = tiles[2 * blockIdx.y];
+  if (e < 0) return;
+  const int row0 = tiles[2 * blockIdx.y + 1], row_end = offsets[e + 1];
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int n0 = blockIdx.x * kTileN;
+  if (tid < kTileM) slot_of[tid] = row0 + tid < row_end ? perm[row0 + tid] : -1;
+  __syncthreads();
+  const TW* we = w + (size_t)e * N * K;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += kStepK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int el = tid + i * 256;
+      const int r = el >> 4, kk = el & 15, k = k0 + kk;
+      const int slot = slot_of[r];
+      float av = 0.f;
+      if (slot >= 0 && k < K) {
+        av = to_f32(a[(size_t)(slot / a_div) * lda + k]);
+        if (scale) av *= scale[slot];
+      }
+      as[kk][r] = av;
+      ws[kk][r] = (n0 + r < N && k < K) ? to_f32(we[(size_t)(n0 + r) * K + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < kStepK; ++kk) {
+      float av[4], wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = as[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wv[j] = ws[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int slot = slot_of[ty * 4 + i];
+    if (slot < 0) continue;
+    const size_t row = plane_rows > 0 ? (size_t)(slot % top) * plane_rows + slot / top : (size_t)slot;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < N) c[row * ldc + n] = from_f32<TC>(acc[i][j]);
+    }
+  }
+}
+
+extern "C" int atoma_route_topk(const float* logits, int ld, int experts, int top, int32_t* ids, float* weights,
+                                int n_tokens, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (experts <= 0 || experts > 1024 || top <= 0 || top > experts || ld < experts) return ATOMA_ERR_SHAPE;
+  hipLaunchKernelGGL(route_topk_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, stream, logits, ld, experts, top, ids,
+                     weights, n_tokens);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+// the most row tiles that n_slots slots of `experts` experts can need
+extern "C" int atoma_route_max_tiles(int n_slots, int experts) {
+  const int full = n_slots / kTileM + experts;
+  return full < n_slots ? full : (n_slots > 0 ? n_slots : 1);
+}
+
+extern "C" int atoma_route_group(const int32_t* ids, int n_slots, int experts, int32_t* perm, int32_t* offsets,
+                                 int32_t* tiles, int max_tiles, hipStream_t stream) {
+  if (n_slots <= 0) return 0;
+  if (experts <= 0 || experts > 1024 || max_tiles < atoma_route_max_tiles(n_slots, experts)) return ATOMA_ERR_SHAPE;
+  hipLaunchKernelGGL(route_group_kernel, dim3(1), dim3(1024), 0, stream, ids, n_slots, experts, perm, offsets, tiles,
+                     max_tiles);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int atoma_expert_gemm(const void* a, int a_dtype, int lda, int a_div, const float* scale, const void* w,
+                                 int w_dtype, void* c, int c_dtype, int ldc, int N, int K, const int32_t* perm,
+                                 const int32_t* offsets, const int32_t* tiles, int max_tiles, int top, int plane_rows,
+                                 hipStream_t stream) {
+  if (max_tiles <= 0 || N <= 0) return 0;
+  if (K <= 0 || lda < K || ldc < N || a_div <= 0 || top <= 0 || max_tiles > 65535) return ATOMA_ERR_SHAPE;
+  dim3 grid((N + kTileN - 1) / kTileN, max_tiles), block(256);
+#define ATOMA_EG(TA, TW, TC)                                                                                       \
+  hipLaunchKernelGGL((expert_gemm_kernel<TA, TW, TC>), grid, block, 0, stream, (const TA*)a, lda, a_div, scale,     \
+                     (const TW*)w, (TC*)c, ldc, N, K, perm, offsets, tiles, top, plane_rows)
+  if (a_dtype == kF32 && w_dtype == kF32 && c_dtype == kF32) ATOMA_EG(float, float, float);
+  else if (a_dtype == kF32 && w_dtype == kBF16 && c_dtype == kF32) ATOMA_EG(float, bf16_t, float);
+  else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kF32) ATOMA_EG(bf16_t, bf16_t, float);
+  else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kBF16) ATOMA_EG(bf16_t, bf16_t, bf16_t);
+  else return ATOMA_ERR_DTYPE;
+#undef ATOMA_EG
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}

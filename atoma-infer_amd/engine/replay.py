@@ -25,7 +25,7 @@ from ..models.model import load_model
 from .step import ModelRunner, StepEntry
 
 REPLAY_PAGE_SIZE = 16       # the engine's default block size ([cache] block_size)
-REPLAY_MAX_LIVE = 16
+REPLAY_MAX_LIVE = 4         # state slots: the most requests that are live at a time
 
 
 def make_runner(model_dir: str, dtype: str, max_tokens: int, page_size: int = REPLAY_PAGE_SIZE,

@@ -485,10 +485,12 @@ def _merge_counters(device: torch.device, needed: int) -> Optional[torch.Tensor]
     return t
 
 
-def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, hd) -> bool:
+def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, hd, sinks=None) -> bool:
     """Run the fast kernels if they take this shape; False sends the caller to the general kernel."""
     page = cache.page_size
     if not page_ok(page) or hd % 16 or not 16 <= hd <= 256:
+        return False
+    if window < 0 or sinks is not None:
         return False
     if q.stride(0) % 8 or q.data_ptr() % 16 or out.stride(0) % 4:
         return False

@@ -48,6 +48,10 @@ HIP_MODULES: Dict[str, Tuple[Sequence[str], Sequence[str]]] = {
     "core": (("elementwise.hip", "attention_generic.hip", "gemm_generic.hip", "sampling.hip"), ()),
     "gemm_bf16": (("gemm_bf16.hip",), ()),
     "microbench": (("microbench.hip",), ()),
+    # mechanisms that only some architectures have; each is compiled when a model first uses it
+    "layer_norms": (("norm_sandwich.hip", "qk_norm_rope.hip"), ()),
+    "delta_rule": (("delta_rule.hip",), ()),
+    "experts": (("experts.hip",), ()),
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}

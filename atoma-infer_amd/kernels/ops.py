@@ -203,12 +203,14 @@ def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[t
 def paged_attention_generic(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, out: torch.Tensor,
                             block_tables: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor,
                             scale: float, window: int, page_size: int, nh: int, nkv: int, hd: int,
-                            slopes: Optional[torch.Tensor] = None) -> None:
+                            slopes: Optional[torch.Tensor] = None, chunk: int = 0,
+                            sinks: Optional[torch.Tensor] = None) -> None:
     """Attention of every token of ``q`` [T, >= nh hd] (row stride free) over its request's cached keys.
 
     Token t belongs to row ``token_seq[t]`` of ``block_tables`` and sits at absolute position ``positions[t]``;
     it sees keys max(0, p - window + 1) .. p (window 0: all).  ``out`` is [T, nh hd].  ``slopes`` (float32 [nh]):
-    head h's score of key j gains ``slopes[h] * (j - p)``.
+    head h's score of key j gains ``slopes[h] * (j - p)``.  ``chunk`` > 0: it sees only keys from (p // chunk) * chunk
+    on.  ``sinks`` (float32 [nh]): the softmax denominator also holds exp(sinks[h]).
     """
     _dev(q, kcache, vcache, out, block_tables, token_seq, positions)
     t = q.shape[0]
@@ -227,10 +229,15 @@ def paged_attention_generic(q: torch.Tensor, kcache: torch.Tensor, vcache: torch
         _dev(slopes)
         _need(slopes.dtype is torch.float32 and slopes.is_contiguous() and slopes.numel() == nh,
               "slopes must be contiguous float32, one per query head")
+    if sinks is not None:
+        _dev(sinks)
+        _need(sinks.dtype is torch.float32 and sinks.is_contiguous() and sinks.numel() == nh,
+              "sinks must be contiguous float32, one per query head")
+    _need(chunk >= 0, "chunk must not be negative")
     _check(core().atoma_paged_attention_generic(
         _p(q), q.stride(0), _p(kcache), _p(vcache), _p(out), out.stride(0), _code(q, "q"), _code(kcache, "cache"),
         _p(block_tables), block_tables.shape[1], _p(token_seq), _p(positions), ctypes.c_float(scale), int(window),
-        page_size, t, nh, nkv, hd, _p(slopes), _stream()), "paged_attention_generic")
+        page_size, t, nh, nkv, hd, _p(slopes), int(chunk), _p(sinks), _stream()), "paged_attention_generic")
 
 
 def swiglu(gu: torch.Tensor, out: Optional[torch.Tensor] = None, block: int = 0) -> torch.Tensor:
@@ -265,6 +272,212 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, out: 
                                      a.stride(0) if m > 1 else k, w.stride(0) if n > 1 else k,
                                      out.stride(0) if m > 1 else n, _stream()), "gemm_generic")
     return out
+
+
+# ------------------------------------------------------------------------------------------------------------
+# mechanisms that only some architectures have: each module is compiled when a model first uses it
+
+_modules = {}
+
+
+def _module(name: str):
+    lib = _modules.get(name)
+    if lib is None:
+        lib = _modules[name] = load_hip_module(name)
+    return lib
+
+
+def _f32(t: torch.Tensor, what: str, n: Optional[int] = None):
+    _need(t.dtype is torch.float32 and t.is_contiguous(), f"{what} must be a contiguous float32 tensor")
+    if n is not None:
+        _need(t.numel() == n, f"{what} has {t.numel()} entries, {n} are needed")
+
+
+def _term(delta: torch.Tensor, t: int, width: int):
+    """(pointer, dtype code, planes, plane stride) of a delta [T, W] or of planes [S, T, W]."""
+    _need(delta.is_contiguous() and tuple(delta.shape[-2:]) == (t, width) and delta.dim() in (2, 3),
+          "a term must be contiguous [T, W] or [planes, T, W] and match resid")
+    planes = delta.shape[0] if delta.dim() == 3 else 1
+    return _p(delta), _code(delta, "term"), planes, ctypes.c_size_t(t * width)
+
+
+def add_normed(resid: torch.Tensor, terms, w_post: torch.Tensor, eps_post: float,
+               w_next: Optional[torch.Tensor] = None, eps_next: float = 0.0,
+               out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """resid += rmsnorm(sum_i scale_i * term_i) * w_post (float32, in place); with ``w_next`` also returns
+    rmsnorm(resid) * w_next in ``out_dtype``.  ``terms``: one or two (tensor, scale) pairs, each tensor [T, W] or
+    planes [S, T, W] (summed), float32 or bfloat16.  Norm weights are float32."""
+    _need(resid.dtype is torch.float32 and resid.dim() == 2 and resid.is_contiguous(), "resid must be float32 [T, W]")
+    t, width = resid.shape
+    _need(1 <= len(terms) <= 2, "one or two terms")
+    _need(width <= 16000, "rows of more than 16,000 columns do not fit the kernel's row buffer")
+    _dev(resid, w_post, w_next, *[d for d, _ in terms])
+    _f32(w_post, "norm weight", width)
+    out = None
+    if w_next is not None:
+        _f32(w_next, "norm weight", width)
+        out = torch.empty((t, width), dtype=out_dtype, device=resid.device)
+    a = _term(terms[0][0], t, width)
+    b = _term(terms[1][0], t, width) if len(terms) > 1 else (_p(None), F32, 0, ctypes.c_size_t(0))
+    _check(_module("layer_norms").atoma_add_normed(
+        _p(resid), *a, ctypes.c_float(terms[0][1]), *b, ctypes.c_float(terms[1][1] if len(terms) > 1 else 0.0),
+        _p(w_post), ctypes.c_float(eps_post), _p(w_next), ctypes.c_float(eps_next), _p(out),
+        _code(out, "out") if out is not None else F32, t, width, _stream()), "add_normed")
+    return out
+
+
+def qk_norm_rope(qk: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, rot_dim: int, wq: torch.Tensor,
+                 wk: torch.Tensor, eps: float, q_out: torch.Tensor, kcache: Optional[torch.Tensor],
+                 vcache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor], page_size: int, nh: int,
+                 nkv: int, hd: int) -> None:
+    """From qk float32 [T, >= (nh + nkv) hd]: q and k normed over their whole projections (weights wq [nh hd],
+    wk [nkv hd]), the first ``rot_dim`` columns of every head rotated in neighbouring pairs by position *
+    inv_freq[i]; q to ``q_out`` [T, nh hd], k into ``kcache`` tiles at ``slot_mapping``; ``vcache`` (optional)
+    receives the k projection as it came."""
+    _dev(qk, positions, inv_freq, wq, wk, q_out, kcache, vcache, slot_mapping)
+    t = qk.shape[0]
+    _need(qk.dtype is torch.float32 and qk.dim() == 2 and qk.stride(1) == 1 and qk.shape[1] >= (nh + nkv) * hd,
+          "qk must be float32 [T, >= (nh + nkv) hd]")
+    _i32(positions, "positions", t)
+    _f32(inv_freq, "inv_freq", rot_dim // 2)
+    _f32(wq, "q norm weight", nh * hd)
+    _f32(wk, "k norm weight", nkv * hd)
+    _need(q_out.dim() == 2 and q_out.stride(1) == 1 and q_out.shape[0] == t and q_out.shape[1] >= nh * hd,
+          "q_out must be [T, nh hd]")
+    cache_code = _code(q_out, "q_out")
+    if kcache is not None:
+        _need(slot_mapping is not None, "a cache write needs slots")
+        _i32(slot_mapping, "slot_mapping", t)
+        pages = kcache.shape[0]
+        _need(kcache.is_contiguous() and tuple(kcache.shape) == (pages, nkv, page_size * hd), "key tiles: bad shape")
+        cache_code = _code(kcache, "cache")
+        if vcache is not None:
+            _need(vcache.is_contiguous() and tuple(vcache.shape) == tuple(kcache.shape)
+                  and vcache.dtype is kcache.dtype, "value tiles must match the key tiles")
+    else:
+        _need(vcache is None, "values without keys")
+    _check(_module("layer_norms").atoma_qk_norm_rope(
+        _p(qk), qk.stride(0), _p(positions), _p(inv_freq), int(rot_dim), _p(wq), _p(wk), ctypes.c_float(eps),
+        _p(q_out), q_out.stride(0), _code(q_out, "q_out"), _p(kcache), _p(vcache), cache_code, _p(slot_mapping),
+        int(page_size), t, nh, nkv, hd, _stream()), "qk_norm_rope")
+
+
+def delta_prepare(proj: torch.Tensor, offsets, heads: int, kv_heads: int, dim: int, vdim: int, taps: int,
+                  token_seq: torch.Tensor, q_start: torch.Tensor, state_slots: torch.Tensor, state: torch.Tensor,
+                  taps_w: torch.Tensor, dt_pre: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor):
+    """The inputs of the gated delta rule for every token (see delta_rule.hip): (q, k, v, beta, decay), all float32,
+    from ``proj`` float32 [T, ld] whose columns ``offsets`` = (q, k, v, b) name; the convolution's state rows of each
+    entry's request are read and then replaced."""
+    _dev(proj, token_seq, q_start, state_slots, state, taps_w, dt_pre, dt_bias, a_log)
+    t = proj.shape[0]
+    s = state_slots.numel()
+    nqk, nv, nd = kv_heads * dim, heads * vdim, heads * dim
+    channels = 2 * nqk + nv
+    off_q, off_k, off_v, off_b = (int(o) for o in offsets)
+    _need(proj.dtype is torch.float32 and proj.dim() == 2 and proj.stride(1) == 1, "proj must be float32 [T, ld]")
+    _need(max(off_q + nqk, off_k + nqk, off_v + nv, off_b + heads) <= proj.shape[1] and min(offsets) >= 0,
+          "the projections' columns do not fit proj")
+    _i32(token_seq, "token_seq", t)
+    _i32(q_start, "q_start", s + 1)
+    _i32(state_slots, "state_slots", s)
+    _need(state.dtype is torch.float32 and state.dim() == 2 and state.is_contiguous()
+          and state.shape[1] == (taps - 1) * channels + heads * vdim * dim, "state: bad shape")
+    _f32(taps_w, "taps", channels * taps)
+    _need(dt_pre.dtype is torch.float32 and dt_pre.is_contiguous() and tuple(dt_pre.shape) == (t, nd), "dt_pre: bad shape")
+    _f32(dt_bias, "dt_bias", nd)
+    _f32(a_log, "A_log", heads)
+    dev = proj.device
+    qn = torch.empty((t, nqk), dtype=torch.float32, device=dev)
+    kn = torch.empty((t, nqk), dtype=torch.float32, device=dev)
+    vn = torch.empty((t, nv), dtype=torch.float32, device=dev)
+    beta = torch.empty((t, heads), dtype=torch.float32, device=dev)
+    decay = torch.empty((t, nd), dtype=torch.float32, device=dev)
+    _check(_module("delta_rule").atoma_delta_prepare(
+        _p(proj), proj.stride(0), off_q, off_k, off_v, off_b, heads, kv_heads, dim, vdim, taps, _p(token_seq),
+        _p(q_start), _p(state_slots), _p(state), ctypes.c_size_t(state.stride(0)), _p(taps_w), _p(dt_pre), _p(dt_bias),
+        _p(a_log), _p(qn), _p(kn), _p(vn), _p(beta), _p(decay), t, s, _stream()), "delta_prepare")
+    return qn, kn, vn, beta, decay
+
+
+def delta_scan(qn, kn, vn, beta, decay, heads: int, kv_heads: int, dim: int, vdim: int, taps: int,
+               q_start: torch.Tensor, state_slots: torch.Tensor, state: torch.Tensor) -> torch.Tensor:
+    """The recurrence over every entry's tokens, from and into the requests' state rows; returns o float32 [T, heads vdim]."""
+    _dev(qn, kn, vn, beta, decay, q_start, state_slots, state)
+    t, s = qn.shape[0], state_slots.numel()
+    nqk, nv, nd = kv_heads * dim, heads * vdim, heads * dim
+    for x, n, what in ((qn, nqk, "q"), (kn, nqk, "k"), (vn, nv, "v"), (beta, heads, "beta"), (decay, nd, "decay")):
+        _need(x.dtype is torch.float32 and x.is_contiguous() and tuple(x.shape) == (t, n), f"{what}: bad shape")
+    _i32(q_start, "q_start", s + 1)
+    _i32(state_slots, "state_slots", s)
+    _need(state.dtype is torch.float32 and state.dim() == 2 and state.is_contiguous()
+          and state.shape[1] == (taps - 1) * (2 * nqk + nv) + heads * vdim * dim, "state: bad shape")
+    o = torch.empty((t, nv), dtype=torch.float32, device=qn.device)
+    _check(_module("delta_rule").atoma_delta_scan(
+        _p(qn), _p(kn), _p(vn), _p(beta), _p(decay), heads, kv_heads, dim, vdim, taps, _p(q_start), _p(state_slots),
+        _p(state), ctypes.c_size_t(state.stride(0)), s, _p(o), _stream()), "delta_scan")
+    return o
+
+
+def delta_out(o: torch.Tensor, gate_pre: torch.Tensor, w: torch.Tensor, eps: float, heads: int, vdim: int,
+              out_dtype: torch.dtype) -> torch.Tensor:
+    """o / sqrt(mean over a head's columns of o^2 + eps) * w * sigmoid(gate_pre), in ``out_dtype``."""
+    _dev(o, gate_pre, w)
+    t = o.shape[0]
+    for x, what in ((o, "o"), (gate_pre, "gate")):
+        _need(x.dtype is torch.float32 and x.is_contiguous() and tuple(x.shape) == (t, heads * vdim), f"{what}: bad shape")
+    _f32(w, "norm weight", vdim)
+    out = torch.empty((t, heads * vdim), dtype=out_dtype, device=o.device)
+    _check(_module("delta_rule").atoma_delta_out(_p(o), _p(gate_pre), _p(w), ctypes.c_float(eps), _p(out),
+                                                 _code(out, "out"), t, heads, vdim, _stream()), "delta_out")
+    return out
+
+
+def route_topk(logits: torch.Tensor, top: int):
+    """(ids int32 [T, top], scores float32 [T, top]): the ``top`` largest sigmoid(logits) of each row."""
+    _dev(logits)
+    _need(logits.dtype is torch.float32 and logits.dim() == 2 and logits.stride(1) == 1, "router logits: float32 [T, E]")
+    t, e = logits.shape
+    ids = torch.empty((t, top), dtype=torch.int32, device=logits.device)
+    scores = torch.empty((t, top), dtype=torch.float32, device=logits.device)
+    _check(_module("experts").atoma_route_topk(_p(logits), logits.stride(0), e, int(top), _p(ids), _p(scores), t,
+                                               _stream()), "route_topk")
+    return ids, scores
+
+
+def route_group(ids: torch.Tensor, experts: int):
+    """Slots (token, choice) ordered by expert: (perm int32 [slots], offsets int32 [experts + 1], tiles int32
+    [max_tiles, 2] of (expert or -1, first place in perm))."""
+    _dev(ids)
+    _i32(ids, "ids")
+    n = ids.numel()
+    lib = _module("experts")
+    max_tiles = int(lib.atoma_route_max_tiles(n, experts))
+    perm = torch.empty(n, dtype=torch.int32, device=ids.device)
+    offsets = torch.empty(experts + 1, dtype=torch.int32, device=ids.device)
+    tiles = torch.empty((max_tiles, 2), dtype=torch.int32, device=ids.device)
+    _check(lib.atoma_route_group(_p(ids), n, experts, _p(perm), _p(offsets), _p(tiles), max_tiles, _stream()),
+           "route_group")
+    return perm, offsets, tiles
+
+
+def expert_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, perm, offsets, tiles, top: int, *,
+                gather: bool, scale: Optional[torch.Tensor] = None, planes: bool = False) -> None:
+    """out[row(slot)] = (scale[slot] * a[src(slot)]) @ w[expert(slot)]^T in float32 arithmetic, for every slot.
+    ``gather``: src is the slot's token (a [T, K]), else the slot (a [slots, K]).  ``planes``: out is [top, T, N]
+    and choice c of token t goes to out[c, t], else out is [slots, N]."""
+    _dev(a, w, out, perm, offsets, tiles, scale)
+    n_slots = perm.numel()
+    e, n, k = w.shape
+    _need(w.is_contiguous() and a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == k, "expert_gemm: a and w do not fit")
+    _need(a.shape[0] * (top if gather else 1) == n_slots, "expert_gemm: rows of a do not fit the slots")
+    _need(out.is_contiguous() and out.numel() == n_slots * n and out.shape[-1] == n, "expert_gemm: bad out")
+    _need(offsets.numel() == e + 1 and tiles.dim() == 2 and tiles.shape[1] == 2, "expert_gemm: bad grouping")
+    if scale is not None:
+        _need(scale.dtype is torch.float32 and scale.is_contiguous() and scale.numel() == n_slots, "expert_gemm: bad scale")
+    _check(_module("experts").atoma_expert_gemm(
+        _p(a), _code(a, "a"), a.stride(0) if a.shape[0] > 1 else k, top if gather else 1, _p(scale), _p(w),
+        _code(w, "w"), _p(out), _code(out, "out"), n, n, k, _p(perm), _p(offsets), _p(tiles), tiles.shape[0], int(top),
+        n_slots // top if planes else 0, _stream()), "expert_gemm")
 
 
 SPLIT_MAX_VOCAB = 262144       # the largest vocabulary whose rows ``sample_packed(split=True)`` cuts into parts

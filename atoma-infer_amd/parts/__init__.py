@@ -2,15 +2,19 @@
 from .base import (Block, CacheSpec, FeedForward, Mixer, Norm, Part, PositionEncoding, StateSpec, WeightSpec,
                    make_part, register_block, register_feed_forward, register_mixer, register_norm,
                    register_position, registered_kinds)
-from .attention import PagedAttention
-from .block import PreNormBlock
+from .attention import PagedAttention, TiedValueAttention
+from .block import PreNormBlock, SandwichBlock
 from .embedding import OutputHead, TokenEmbedding
+from .experts import RoutedExperts
 from .feed_forward import SwiGLU
 from .linear import linear
 from .norm import RMSNorm
+from .parallel import ParallelMixer
 from .position import NoPosition, RotaryEncoding
+from .recurrent import GatedDeltaRule
 
 __all__ = ["Block", "CacheSpec", "FeedForward", "Mixer", "Norm", "Part", "PositionEncoding", "StateSpec",
            "WeightSpec", "make_part", "register_block", "register_feed_forward", "register_mixer", "register_norm",
            "register_position", "registered_kinds", "PagedAttention", "PreNormBlock", "OutputHead",
-           "TokenEmbedding", "SwiGLU", "linear", "RMSNorm", "NoPosition", "RotaryEncoding"]
+           "TokenEmbedding", "SwiGLU", "linear", "RMSNorm", "NoPosition", "RotaryEncoding", "TiedValueAttention",
+           "SandwichBlock", "RoutedExperts", "ParallelMixer", "GatedDeltaRule"]

@@ -29,7 +29,7 @@ from .linear import as_tensor, linear, linear_delta
 class PagedAttention(Mixer):
     def __init__(self, width: int, num_heads: int, num_kv_heads: int, head_size: int,
                  position: Optional[PositionEncoding] = None, window: Optional[int] = None,
-                 scale: Optional[float] = None):
+                 scale: Optional[float] = None, chunk: Optional[int] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads cannot be grouped over {num_kv_heads} KV heads")
         # every multiple of 8 up to 256, as the reference's kernels take (csrc/src/lib.rs:136-143, 790)
@@ -38,9 +38,14 @@ class PagedAttention(Mixer):
                              f"from 8 to 256")
         if window is not None and window <= 0:
             raise ValueError("window must be positive")
+        if chunk is not None and (chunk <= 0 or window is not None):
+            raise ValueError("chunk must be positive, and a layer has a window or chunks, not both")
         self.width, self.nh, self.nkv, self.hd = int(width), int(num_heads), int(num_kv_heads), int(head_size)
         self.position = position
         self.window = window
+        # chunk c: the token at p sees keys (p // c) * c .. p only, chunks counted from the request's first position
+        self.chunk = chunk
+        self.sinks: Optional[torch.Tensor] = None       # float32 [heads]: exp(sinks[h]) joins the softmax denominator
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd)
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
@@ -98,7 +103,7 @@ class PagedAttention(Mixer):
         kernels, built once per step on the host and shipped with the step's metadata.  ``bucket_tokens`` is None, or
         for a step that only decodes the context length its plan must serve (a multiple of the runner's bucket)."""
         from ..kernels import attention_bf16
-        if self.slopes is not None:
+        if self.slopes is not None or self.chunk or self.sinks is not None:
             return None          # scores with a bias take the general kernel, which needs no plan
         if cache_dtype is torch.bfloat16 and self.hd % 16:
             import warnings
@@ -113,13 +118,19 @@ class PagedAttention(Mixer):
                           f"multiple of 16 tokens ([cache] block_size = 16, 32, 64, ...)", stacklevel=2)
         if cache_dtype is not torch.bfloat16 or not attention_bf16.page_ok(page_size):
             return None
-        group, window, nkv = self.nh // self.nkv, self.window or 0, self.nkv
-        cus = torch.cuda.get_device_properties(self.w_qkv.device).multi_processor_count
+        group, window, nkv = self.nh // self.nkv, self.span, self.nkv
+        cus = torch.cuda.get_device_properties(self.w_o.device).multi_processor_count
         return (attention_bf16.plan_key(group, window, nkv, self.hd),
                 lambda starts, counts, bucket: attention_bf16.build_tasks(
                     starts, counts, group, window, bucket, kv_heads=nkv,
                     max_waves=attention_bf16.max_waves_for(self.hd),
                     row_tiles=attention_bf16.max_row_tiles_for(self.hd), head_size=self.hd, compute_units=cus))
+
+    @property
+    def span(self) -> int:
+        """The mask as the matrix-core kernels and their planner take it: w > 0 a window of the last w keys, -c < 0
+        chunks of c positions, 0 all keys."""
+        return -self.chunk if self.chunk else (self.window or 0)
 
     # -- execution ------------------------------------------------------------------------------------
     accepts_begun = True
@@ -171,12 +182,89 @@ class PagedAttention(Mixer):
     def attend(self, q, k_cache, v_cache, out, ctx, cache) -> None:
         if self.slopes is None and q.dtype is torch.bfloat16 and k_cache.dtype is torch.bfloat16:
             from ..kernels import attention_bf16
-            if attention_bf16.try_attention(q, k_cache, v_cache, out, ctx, cache, self.scale, self.window or 0,
-                                            self.nh, self.nkv, self.hd):
+            if attention_bf16.try_attention(q, k_cache, v_cache, out, ctx, cache, self.scale, self.span,
+                                            self.nh, self.nkv, self.hd, self.sinks):
                 return
         ops.paged_attention_generic(q, k_cache, v_cache, out, cache.block_tables, ctx.token_seq, ctx.positions,
                                     self.scale, self.window or 0, cache.page_size, self.nh, self.nkv, self.hd,
-                                    self.slopes)
+                                    self.slopes, self.chunk or 0, self.sinks)
+
+
+class TiedValueAttention(PagedAttention):
+    """Attention whose values are its keys: ``v = W_k x`` as projected, while the keys go on through a norm and the
+    rotation.  There is no value projection.
+
+    * q and k are normed over their whole projections (all heads at once) with plain weights ``q.norm``
+      [heads * head_size] and ``k.norm`` [kv_heads * head_size], before the rotation;
+    * the first ``rotary_dim`` columns of every head are rotated in neighbouring pairs (2i, 2i + 1) by
+      position * base^(-2i / rotary_dim), angles in float32, for any position (no table);
+    * optional chunks and one learned sink per head (tensor ``sink``), see ``PagedAttention``.
+
+    Tensors: ``q``, ``k``, ``o`` ([out, in]), ``q.norm``, ``k.norm``, ``sink``.
+    """
+
+    def __init__(self, width: int, num_heads: int, num_kv_heads: int, head_size: int, scale: float, norm_eps: float,
+                 rotary_base: float, rotary_dim: int, chunk: Optional[int] = None, window: Optional[int] = None,
+                 sink: bool = True):
+        super().__init__(width, num_heads, num_kv_heads, head_size, None, window, scale, chunk)
+        if head_size % 2 or rotary_dim % 2 or not 0 <= rotary_dim <= head_size or rotary_dim > 256:
+            raise ValueError(f"rotary_dim {rotary_dim} must be even, at most the head size {head_size} and at most 256")
+        self.norm_eps, self.rotary_base, self.rotary_dim, self.has_sink = float(norm_eps), float(rotary_base), \
+            int(rotary_dim), bool(sink)
+        self.w_qk = self.q_norm = self.k_norm = self.inv_freq = None
+
+    def graph_safe(self) -> bool:
+        return True
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        q, kv = self.nh * self.hd, self.nkv * self.hd
+        specs = {"q": WeightSpec((q, self.width)), "k": WeightSpec((kv, self.width)),
+                 "q.norm": WeightSpec((q,), "norm"), "k.norm": WeightSpec((kv,), "norm"),
+                 "o": WeightSpec((self.width, q))}
+        if self.has_sink:
+            specs["sink"] = WeightSpec((self.nh,), "linear", std=1.0)
+        return specs
+
+    def load(self, get, device, act_dtype) -> None:
+        ws = [get("q"), get("k")]
+        dt = ws[0].dtype if ws[0].dtype is ws[1].dtype else torch.float32
+        self.w_qk = torch.cat([w.to(device=device, dtype=dt) for w in ws], dim=0).contiguous()
+        self.w_o = get("o").to(device).contiguous()
+        f32 = dict(device=device, dtype=torch.float32)
+        self.q_norm, self.k_norm = get("q.norm").to(**f32).contiguous(), get("k.norm").to(**f32).contiguous()
+        self.sinks = get("sink").to(**f32).contiguous() if self.has_sink else None
+        # base^(-2i / dims) in double precision, rounded once to float32
+        i = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
+        self.inv_freq = torch.pow(torch.tensor(self.rotary_base, dtype=torch.float64),
+                                  -2.0 * i / max(self.rotary_dim, 1)).to(**f32).contiguous()
+        self.act_dtype = act_dtype
+        self.w_o_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_o.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            self.w_o_tiled = gemm_bf16.tile_copies_resid(self.w_o)
+
+    def device_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_qk, self.w_o))
+
+    accepts_begun = False
+    takes_sink = False
+
+    def forward(self, x, ctx, cache, sink=None):
+        nh, nkv, hd = self.nh, self.nkv, self.hd
+        t = x.shape[0]
+        writes = cache.writable
+        if not writes:
+            raise NotImplementedError("tied-value attention reads only a cache of its own")
+        w = self.w_qk
+        # the projection leaves in float32: the norm over it and the rotation are float32 work
+        qk = linear(x, w, torch.float32)
+        q = torch.empty((t, nh * hd), dtype=x.dtype, device=x.device)
+        ops.qk_norm_rope(qk, ctx.positions, self.inv_freq, self.rotary_dim, self.q_norm, self.k_norm, self.norm_eps, q,
+                         cache.k, cache.v, cache.slot_mapping, cache.page_size, nh, nkv, hd)
+        out = torch.empty((t, nh * hd), dtype=x.dtype, device=x.device)
+        self.attend(q, cache.k, cache.v, out, ctx, cache)
+        return linear_delta(out, self.w_o, None, self.w_o_tiled)
 
 
 register_mixer("attention", PagedAttention)
+register_mixer("tied_value_attention", TiedValueAttention)

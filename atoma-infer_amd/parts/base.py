@@ -20,20 +20,35 @@ from typing import Callable, Dict, Optional, Tuple
 import torch
 
 
+#: in a ``WeightSpec``'s shape: a size that the checkpoint decides (the random-weights writer takes ``DEFAULT_FREE``)
+FREE = -1
+DEFAULT_FREE = 16
+
+
 @dataclasses.dataclass(frozen=True)
 class WeightSpec:
     """One checkpoint tensor: its shape, and how the random-weights writer fills it.
 
-    ``init``: "linear" and "embedding" draw N(0, 0.02); "norm" is 1 (plus N(0, norm_jitter) on request);
-    "int_table" draws integers in [0, high).  Integer tables are kept as int32 on the device.
+    ``init``: "linear" and "embedding" draw N(mean, std), by default N(0, 0.02); "norm" is 1 (plus N(0, norm_jitter)
+    on request); "int_table" draws integers in [0, high).  Integer tables are kept as int32 on the device.
     """
     shape: Tuple[int, ...]
     init: str = "linear"
     high: int = 0
+    mean: float = 0.0
+    std: float = 0.02
 
     @property
     def is_int(self) -> bool:
         return self.init == "int_table"
+
+    def fits(self, shape) -> bool:
+        """Whether a stored tensor of ``shape`` is what this spec describes (a ``FREE`` size takes any)."""
+        return len(shape) == len(self.shape) and all(w == FREE or w == g for w, g in zip(self.shape, shape))
+
+    @property
+    def drawn_shape(self) -> Tuple[int, ...]:
+        return tuple(DEFAULT_FREE if w == FREE else w for w in self.shape)
 
 
 @dataclasses.dataclass(frozen=True)
@@ -99,6 +114,14 @@ class Part:
         host or waits for the device says False, the default; a model that holds such a part runs every step
         directly."""
         return False
+
+
+@dataclasses.dataclass
+class WeightedSum:
+    """What a mixer of several branches hands to the norm behind it: ``sum_i scale_i * tensor_i``, not yet added up.
+    Each tensor is a delta [T, W] or float32 planes [S, T, W]; the norm's kernel scales and sums them in float32, in
+    the order of the list."""
+    terms: list
 
 
 @dataclasses.dataclass

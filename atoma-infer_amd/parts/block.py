@@ -3,10 +3,14 @@
 ``PreNormBlock``: ``h = x + mixer(norm1(x))``, ``y = h + ffn(norm2(h))`` (models/src/llama.rs:393-410).  The residual
 stream is float32; each sum is fused with the norm that follows it, so a block receives the previous block's
 output as a pending ``delta`` and returns its own.
+
+``SandwichBlock``: a norm before and a norm behind each sublayer, ``h = x + norm1b(mixer(norm1(x)))``,
+``y = h + norm2b(ffn(norm2(h)))``; the feed-forward half may be absent.  One kernel norms a sublayer's output, adds
+it to the stream and applies the norm that reads the stream next.
 """
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
 
 from .base import Begun, Block, FeedForward, Mixer, Norm, WeightSpec, register_block
 from .linear import Normed, ResidualSink
@@ -65,4 +69,61 @@ class PreNormBlock(Block):
         return self.feed_forward.forward(x, ctx)
 
 
+def _join(prefix: str, rel: str) -> str:
+    return f"{prefix}.{rel}" if prefix and rel else prefix or rel
+
+
+class SandwichBlock(Block):
+    """``norms`` = (before the mixer, behind it, before the feed-forward, behind it); the last two and the
+    feed-forward are None for a layer that has the mixer only.  ``names``: the children's prefixes below the
+    layer's, in the order (norms..., mixer, feed-forward); a norm whose tensor carries its whole name has prefix ""."""
+
+    def __init__(self, norms, mixer: Mixer, feed_forward: Optional[FeedForward] = None,
+                 names=("", "", "", "", "mix", "mlp")):
+        self.norm1, self.norm1b, self.norm2, self.norm2b = norms
+        self.mixer, self.feed_forward = mixer, feed_forward
+        if (feed_forward is None) != (self.norm2 is None) or (feed_forward is None) != (self.norm2b is None):
+            raise ValueError("the feed-forward and its two norms come together or not at all")
+        self.names = tuple(names)
+
+    def _children(self):
+        parts = (self.norm1, self.norm1b, self.norm2, self.norm2b, self.mixer, self.feed_forward)
+        return [(n, p) for n, p in zip(self.names, parts) if p is not None]
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {_join(n, k): ws for n, part in self._children() for k, ws in part.weight_specs().items()}
+
+    def load(self, get, device, act_dtype) -> None:
+        for n, part in self._children():
+            part.load(lambda rel, _n=n: get(_join(_n, rel)), device, act_dtype)
+
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe() for _, part in self._children())
+
+    def device_bytes(self) -> int:
+        return sum(part.device_bytes() for _, part in self._children())
+
+    fuses_next_norm = True
+
+    def entry_norm(self):
+        return self.norm1
+
+    def forward(self, resid, delta, ctx, cache, next_norm=None):
+        if isinstance(delta, Normed):
+            if delta.norm is not self.norm1:
+                raise RuntimeError("a finished norm reached another norm than the one it was made for")
+            x = delta.data
+        else:
+            x = self.norm1.add_norm(resid, delta)
+        a = self.mixer.forward(x, ctx, cache)
+        if self.feed_forward is None:
+            x = self.norm1b.add_normed(resid, a, next_norm)
+        else:
+            x = self.norm1b.add_normed(resid, a, self.norm2)
+            f = self.feed_forward.forward(x, ctx)
+            x = self.norm2b.add_normed(resid, f, next_norm)
+        return Normed(x, next_norm) if next_norm is not None else None
+
+
 register_block("pre_norm", PreNormBlock)
+register_block("sandwich", SandwichBlock)

@@ -16,18 +16,18 @@ from .linear import linear
 
 
 class TokenEmbedding(Part):
-    def __init__(self, vocab_size: int, width: int):
-        self.vocab_size, self.width = int(vocab_size), int(width)
+    def __init__(self, vocab_size: int, width: int, name: str = "weight"):
+        self.vocab_size, self.width, self.name = int(vocab_size), int(width), str(name)
         self.weight: Optional[torch.Tensor] = None
 
     def graph_safe(self) -> bool:
         return True
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {"weight": WeightSpec((self.vocab_size, self.width), "embedding")}
+        return {self.name: WeightSpec((self.vocab_size, self.width), "embedding")}
 
     def load(self, get, device, act_dtype) -> None:
-        self.weight = get("weight").to(device).contiguous()
+        self.weight = get(self.name).to(device).contiguous()
 
     def device_bytes(self) -> int:
         return 0  # a step reads only the rows of its tokens
@@ -42,8 +42,8 @@ class TokenEmbedding(Part):
 
 
 class OutputHead(Part):
-    def __init__(self, width: int, vocab_size: int, tied_to: Optional[TokenEmbedding] = None):
-        self.width, self.vocab_size, self.tied_to = int(width), int(vocab_size), tied_to
+    def __init__(self, width: int, vocab_size: int, tied_to: Optional[TokenEmbedding] = None, name: str = "weight"):
+        self.width, self.vocab_size, self.tied_to, self.name = int(width), int(vocab_size), tied_to, str(name)
         self.weight: Optional[torch.Tensor] = None
         self.tiled = None
 
@@ -51,10 +51,10 @@ class OutputHead(Part):
         return True
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {} if self.tied_to is not None else {"weight": WeightSpec((self.vocab_size, self.width))}
+        return {} if self.tied_to is not None else {self.name: WeightSpec((self.vocab_size, self.width))}
 
     def load(self, get, device, act_dtype) -> None:
-        self.weight = self.tied_to.weight if self.tied_to is not None else get("weight").to(device).contiguous()
+        self.weight = self.tied_to.weight if self.tied_to is not None else get(self.name).to(device).contiguous()
         # a second copy in the order the streaming kernel's waves read it, for steps of few rows (the row-major one
         # serves the embedding's gather and the products of many rows)
         self.tiled = None

@@ -10,23 +10,26 @@ from typing import Dict, Optional
 import torch
 
 from ..kernels import ops
-from .base import Begun, Norm, WeightSpec, register_norm
+from .base import Begun, Norm, WeightedSum, WeightSpec, register_norm
 
 
 class RMSNorm(Norm):
-    def __init__(self, width: int, eps: float):
-        self.width, self.eps = int(width), float(eps)
+    def __init__(self, width: int, eps: float, name: str = "weight"):
+        # ``name``: the tensor's name below the part's prefix ("weight" as checkpoints of the Llama family have it)
+        self.width, self.eps, self.name = int(width), float(eps), str(name)
         self.weight: Optional[torch.Tensor] = None
+        self.weight_f32: Optional[torch.Tensor] = None
         self.act_dtype = torch.float32
 
     def graph_safe(self) -> bool:
         return True
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {"weight": WeightSpec((self.width,), "norm")}
+        return {self.name: WeightSpec((self.width,), "norm")}
 
     def load(self, get, device, act_dtype) -> None:
-        self.weight = get("weight").to(device).contiguous()
+        self.weight = get(self.name).to(device).contiguous()
+        self.weight_f32 = self.weight.to(torch.float32)
         self.act_dtype = act_dtype
 
     def device_bytes(self) -> int:
@@ -34,6 +37,16 @@ class RMSNorm(Norm):
 
     def add_norm(self, resid, delta, rows=None):
         return ops.add_rmsnorm(resid, delta, self.weight, self.eps, self.act_dtype, rows)
+
+    def add_normed(self, resid, delta, next_norm=None):
+        """``resid += self(delta)`` (in place): this norm stands behind a sublayer, whose output ``delta`` (a tensor,
+        float32 planes or a ``WeightedSum`` of up to two such) it norms before the sum.  With ``next_norm`` (an
+        RMSNorm) the same kernel also returns ``next_norm(resid)`` in the activation dtype."""
+        terms = delta.terms if isinstance(delta, WeightedSum) else [(delta, 1.0)]
+        if next_norm is None:
+            return ops.add_normed(resid, terms, self.weight_f32, self.eps)
+        return ops.add_normed(resid, terms, self.weight_f32, self.eps, next_norm.weight_f32, next_norm.eps,
+                              next_norm.act_dtype)
 
     # the norm begun by its neighbours (bfloat16 steps of at most 16 rows): see kernels/gemm_bf16.py; with many rows
     # the library adds its product to the residual rows itself, and the norm reads them once

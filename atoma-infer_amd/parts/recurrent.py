@@ -1,0 +1,122 @@
+"""Recurrent mixers: a state of fixed size per request in place of a cache that grows.
+
+``GatedDeltaRule``: per head a float32 matrix S [dim, vdim] that every token decays, corrects and reads,
+
+    S <- diag(g) S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q,
+
+* q, k (``kv_heads`` heads of ``dim``) and v (``heads`` heads of ``vdim``) are projections of the input that pass a
+  causal depthwise convolution over time (``taps`` taps, the last one the current token's, zeros before the
+  request's start) and SiLU; q and k are then scaled to unit length per head (x / sqrt(sum x^2 + 1e-6)), q also by
+  dim^-1/2; head h reads q/k head h // (heads / kv_heads);
+* beta = sigmoid(W_b x), one per head;
+* g = exp(-exp(A_log[h]) * softplus(W_a2 W_a1 x + dt_bias)), one per head and key channel;
+* the output: o normed per head over vdim (RMS, weight ``norm`` [vdim] shared by the heads), times
+  sigmoid(W_g2 W_g1 x), then W_o.
+
+What is carried from token to token, the state of a request, is S and the last ``taps - 1`` inputs of the
+convolution, all float32: one row of the state tensor, [taps - 1][conv channels] followed by [heads][vdim][dim].
+Decays, gates of the recurrence, unit lengths and the recurrence itself are float32 in both dtypes; the
+projections run in the activation dtype with float32 sums and leave unrounded.
+
+Tensors ([out, in]): ``q``, ``k``, ``v``, ``b``, ``a1``, ``a2``, ``g1``, ``g2``, ``o``; ``q.conv``, ``k.conv``,
+``v.conv`` [channels, taps]; ``A_log`` [heads]; ``dt_bias`` [heads * dim]; ``norm`` [vdim].
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import FREE, Mixer, StateSpec, WeightSpec, register_mixer
+from .linear import linear, linear_delta
+
+
+class GatedDeltaRule(Mixer):
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, taps: int, norm_eps: float,
+                 decay_rank: Optional[int] = None, gate_rank: Optional[int] = None):
+        # the inner sizes of the two low-rank maps (a1/a2 and g1/g2) are the checkpoint's: None takes whatever
+        # the tensors have (the random-weights mode then draws ``DEFAULT_RANK``)
+        if heads % kv_heads:
+            raise ValueError(f"{heads} heads cannot be grouped over {kv_heads} q/k heads")
+        if not 0 < dim <= 256:
+            raise ValueError(f"key size {dim} is not supported: the recurrence's kernel takes up to 256")
+        if taps < 1:
+            raise ValueError("the convolution needs at least the current token's tap")
+        self.width, self.heads, self.kv_heads, self.dim, self.vdim = int(width), int(heads), int(kv_heads), int(dim), int(vdim)
+        self.taps, self.norm_eps = int(taps), float(norm_eps)
+        self.decay_rank = int(decay_rank) if decay_rank else None
+        self.gate_rank = int(gate_rank) if gate_rank else None
+        self.nqk, self.nv, self.nd = self.kv_heads * self.dim, self.heads * self.vdim, self.heads * self.dim
+        self.channels = 2 * self.nqk + self.nv
+        # columns of the fused first projection: q, k, v, b, then a1 and g1 (placed at load time)
+        self.off_q, self.off_k, self.off_v = 0, self.nqk, 2 * self.nqk
+        self.off_b = self.off_v + self.nv
+        self.off_a1 = self.off_b + self.heads
+        self.off_g1 = None
+        self.w_in = self.w_a2 = self.w_g2 = self.w_o = self.w_o_tiled = None
+        self.taps_w = self.a_log = self.dt_bias = self.norm_w = None
+
+    def graph_safe(self) -> bool:
+        return True     # the kernels take entries, slots and lengths from the step's device tensors
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        w, t = self.width, self.taps
+        ra, rg = self.decay_rank or FREE, self.gate_rank or FREE
+        return {"q": WeightSpec((self.nqk, w)), "q.conv": WeightSpec((self.nqk, t), std=0.5),
+                "k": WeightSpec((self.nqk, w)), "k.conv": WeightSpec((self.nqk, t), std=0.5),
+                "v": WeightSpec((self.nv, w)), "v.conv": WeightSpec((self.nv, t), std=0.5),
+                "b": WeightSpec((self.heads, w), std=0.1), "A_log": WeightSpec((self.heads,), std=0.5, mean=-1.0),
+                "norm": WeightSpec((self.vdim,), "norm"),
+                "a1": WeightSpec((ra, w), std=0.1), "a2": WeightSpec((self.nd, ra), std=0.3),
+                "dt_bias": WeightSpec((self.nd,), std=1.0, mean=-2.0),
+                "g1": WeightSpec((rg, w), std=0.1), "g2": WeightSpec((self.nv, rg), std=0.3),
+                "o": WeightSpec((w, self.nv))}
+
+    def state_spec(self) -> StateSpec:
+        return StateSpec(((self.taps - 1) * self.channels + self.heads * self.vdim * self.dim,), "float32")
+
+    def load(self, get, device, act_dtype) -> None:
+        ws = [get(n) for n in ("q", "k", "v", "b", "a1", "g1")]
+        self.decay_rank, self.gate_rank = ws[4].shape[0], ws[5].shape[0]
+        self.off_g1 = self.off_a1 + self.decay_rank
+        dt = ws[0].dtype if all(w.dtype is ws[0].dtype for w in ws) else torch.float32
+        rows = sum(w.shape[0] for w in ws)
+        pad = (-rows) % 64      # whole tiles for the matrix-core products
+        parts = [w.to(device=device, dtype=dt) for w in ws]
+        if pad:
+            parts.append(torch.zeros((pad, self.width), dtype=dt, device=device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        self.w_a2, self.w_g2 = get("a2").to(device).contiguous(), get("g2").to(device).contiguous()
+        if self.w_a2.shape[1] != self.decay_rank or self.w_g2.shape[1] != self.gate_rank:
+            raise ValueError(f"the halves of a low-rank map do not fit: a1 {tuple(ws[4].shape)} and a2 "
+                             f"{tuple(self.w_a2.shape)}, g1 {tuple(ws[5].shape)} and g2 {tuple(self.w_g2.shape)}")
+        self.w_o = get("o").to(device).contiguous()
+        f32 = dict(device=device, dtype=torch.float32)
+        self.taps_w = torch.cat([get(n + ".conv").to(**f32) for n in ("q", "k", "v")], dim=0).contiguous()
+        self.a_log, self.dt_bias = get("A_log").to(**f32).contiguous(), get("dt_bias").to(**f32).contiguous()
+        self.norm_w = get("norm").to(**f32).contiguous()
+        self.w_o_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_o.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            self.w_o_tiled = gemm_bf16.tile_copies_resid(self.w_o)
+
+    def device_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_a2, self.w_g2, self.w_o))
+
+    def forward(self, x, ctx, cache):
+        state = cache.state
+        proj = linear(x, self.w_in, torch.float32)
+        # the second halves of the two low-rank maps read their slices of the float32 projection as they are
+        dt_pre = linear(proj[:, self.off_a1: self.off_a1 + self.decay_rank], self.w_a2, torch.float32)
+        gate_pre = linear(proj[:, self.off_g1: self.off_g1 + self.gate_rank], self.w_g2, torch.float32)
+        qn, kn, vn, beta, decay = ops.delta_prepare(
+            proj, (self.off_q, self.off_k, self.off_v, self.off_b), self.heads, self.kv_heads, self.dim, self.vdim,
+            self.taps, ctx.token_seq, ctx.q_start, ctx.state_slots, state, self.taps_w, dt_pre, self.dt_bias, self.a_log)
+        o = ops.delta_scan(qn, kn, vn, beta, decay, self.heads, self.kv_heads, self.dim, self.vdim, self.taps,
+                           ctx.q_start, ctx.state_slots, state)
+        y = ops.delta_out(o, gate_pre, self.norm_w, self.norm_eps, self.heads, self.vdim, x.dtype)
+        return linear_delta(y, self.w_o, None, self.w_o_tiled)
+
+
+register_mixer("gated_delta_rule", GatedDeltaRule)

@@ -110,7 +110,7 @@ def check_checkpoint(spec, ckpt: Checkpoint) -> None:
     for n, ws in want.items():
         if n not in have:
             continue
-        if tuple(ckpt.shape(n)) != tuple(ws.shape):
+        if not ws.fits(tuple(ckpt.shape(n))):
             wrong_shape.append((n, tuple(ckpt.shape(n)), tuple(ws.shape)))
         is_float = ckpt.dtype(n).is_floating_point
         if ws.is_int and is_float:

@@ -1,6 +1,6 @@
 """Random-weights mode: write a model folder from a configuration and a seed.
 
-The reference has no such mode.  Linears and embeddings are drawn from N(0, 0.02); norm weights are 1, or
+The reference has no such mode.  Linears and embeddings are drawn from N(0, 0.02) unless their part asks for another mean and spread; norm weights are 1, or
 1 + N(0, norm_jitter).  Every tensor has a generator of its own, keyed by (seed, tensor name), so a tensor's
 values do not depend on which other tensors the model has or on the order of writing.
 """
@@ -33,13 +33,13 @@ def random_tensor(name: str, ws: WeightSpec, seed: int, dtype: torch.dtype, norm
                   ) -> torch.Tensor:
     g = _generator(seed, name)
     if ws.init in ("linear", "embedding"):
-        t = torch.randn(ws.shape, generator=g, dtype=torch.float32) * 0.02
+        t = torch.randn(ws.drawn_shape, generator=g, dtype=torch.float32) * ws.std + ws.mean
     elif ws.init == "norm":
-        t = torch.ones(ws.shape, dtype=torch.float32)
+        t = torch.ones(ws.drawn_shape, dtype=torch.float32)
         if norm_jitter:
-            t += torch.randn(ws.shape, generator=g, dtype=torch.float32) * norm_jitter
+            t += torch.randn(ws.drawn_shape, generator=g, dtype=torch.float32) * norm_jitter
     elif ws.init == "int_table":
-        return torch.randint(0, max(ws.high, 1), ws.shape, generator=g, dtype=torch.int32)
+        return torch.randint(0, max(ws.high, 1), ws.drawn_shape, generator=g, dtype=torch.int32)
     else:
         raise ValueError(f"tensor '{name}': unknown init '{ws.init}'")
     return t.to(dtype)
