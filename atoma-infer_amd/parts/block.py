@@ -113,6 +113,10 @@ class SandwichBlock(Block):
             if delta.norm is not self.norm1:
                 raise RuntimeError("a finished norm reached another norm than the one it was made for")
             x = delta.data
+        elif isinstance(delta, Begun):
+            if delta.norm is not self.norm1:
+                raise RuntimeError("a begun norm reached another norm than the one it was begun for")
+            x = delta.tensor()
         else:
             x = self.norm1.add_norm(resid, delta)
         a = self.mixer.forward(x, ctx, cache)
