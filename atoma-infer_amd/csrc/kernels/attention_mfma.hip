@@ -19,7 +19,10 @@
 //   S^T[key, row] = K[key, :] . Q[row, :]     K page rows are the A operand straight from global memory,
 //                                             Q the B operand, kept in registers for the whole task;
 //   online softmax down the keys of each row in float32 (exp2 with the scale folded in), masked by the row's
-//   own position and window (bottom-right aligned causal mask, csrc/kernels/mask.h:171-192);
+//   own position and window (bottom-right aligned causal mask, csrc/kernels/mask.h:171-192); a negative window -c
+//   means chunks of c positions instead: the row at p sees keys (p / c) * c .. p.  With sinks (one float32 per query
+//   head) exp(sink) joins a row's softmax denominator, once, where the row's output is written: by the task that
+//   walked all its keys, or by whoever merges its chunks;
 //   O^T[d, row] += V^T[d, key] . P^T[key, row]  S^T's accumulator layout is already the B operand layout, so
 //                                             P goes from registers to the MFMA as bfloat16 without a
 //                                             transpose, and V^T is how the cache stores values.
@@ -109,7 +112,7 @@ __device__ __forceinline__ float load_through1(const float* p) {
 template <int BATCH>
 __device__ __forceinline__ void merge_parts(const float* __restrict__ part_o, const float* __restrict__ part_lse,
                                             uint16_t* __restrict__ out, int out_stride, const Task& comb, int kvh,
-                                            int nh, int nkv, int lane) {
+                                            int nh, int nkv, int lane, const float* __restrict__ sinks) {
   constexpr int Q = HD / 4;                        // pieces of four values in a row
   const int g = nh / nkv;
   const size_t part_stride = (size_t)nkv * 32;     // rows between two parts of the same (KV head, row)
@@ -151,6 +154,13 @@ __device__ __forceinline__ void merge_parts(const float* __restrict__ part_o, co
       }
       m = mb;
     }
+    if (sinks != nullptr && wsum > 0.f) {
+      const float s2 = sinks[kvh * g + hq] * kLog2e;
+      const float m_f = fmaxf(m, s2);
+      const float corr = __builtin_amdgcn_exp2f(m - m_f);
+      wsum = wsum * corr + __builtin_amdgcn_exp2f(s2 - m_f);
+      acc.x *= corr, acc.y *= corr, acc.z *= corr, acc.w *= corr;
+    }
     const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
     uint2 pk;
     pk.x = (uint32_t)f32_to_bf16_bits(acc.x * inv) | ((uint32_t)f32_to_bf16_bits(acc.y * inv) << 16);
@@ -180,7 +190,8 @@ attention_mfma_kernel(const Task* __restrict__ tasks, int n_tasks, int nkv, cons
                       int q_stride, int nh, const int32_t* __restrict__ block_tables, int max_blocks, int window,
                       const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                       uint16_t* __restrict__ out, int out_stride, float* __restrict__ part_o,
-                      float* __restrict__ part_lse, float scale, int32_t* __restrict__ counters) {
+                      float* __restrict__ part_lse, float scale, int32_t* __restrict__ counters,
+                      const float* __restrict__ sinks) {
   // (the arguments come in the order in which a wave needs them: the first fourteen words, up to kcache, are in
   // scalar registers when the wave starts, the others are fetched from memory, a trip that the task record, the
   // queries, the page numbers and the first keys need not wait for)
@@ -220,6 +231,7 @@ attention_mfma_kernel(const Task* __restrict__ tasks, int n_tasks, int nkv, cons
     trow[t] = row_ok[t] ? task.tok_base + tok : 0;
     p_row[t] = row_ok[t] ? task.pos0 + tok : -1;
     lo_row[t] = (window > 0 && p_row[t] - window + 1 > 0) ? p_row[t] - window + 1 : 0;
+    if (window < 0 && p_row[t] > 0) lo_row[t] = (p_row[t] / -window) * -window;
     head[t] = kvh * g + (row_ok[t] ? hq : 0);
   }
   // a piece without a live row is skipped altogether (the same for all lanes)
@@ -476,6 +488,17 @@ attention_mfma_kernel(const Task* __restrict__ tasks, int n_tasks, int nkv, cons
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
       if (!row_ok[t]) continue;
+      if (sinks != nullptr && l[t] > 0.f) {
+        // (m is in units of the scaled score times log2 e, the sink a natural logarithm)
+        const float s2 = sinks[head[t]] * kLog2e;
+        const float m_f = fmaxf(m[t], s2);
+        const float corr = __builtin_amdgcn_exp2f(m[t] - m_f);
+        l[t] = l[t] * corr + __builtin_amdgcn_exp2f(s2 - m_f);
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[t][dt][i] *= corr;
+      }
       const float inv = l[t] > 0.f ? 1.0f / l[t] : 0.f;
       uint16_t* op = out + (size_t)trow[t] * out_stride + (size_t)head[t] * HD;
 #pragma unroll
@@ -531,7 +554,7 @@ attention_mfma_kernel(const Task* __restrict__ tasks, int n_tasks, int nkv, cons
       if (before + 1 == comb.n_parts) {
         if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
         // (a wave a task: the launches of decoded tokens alone, which have registers to spare)
-        merge_parts<(KSPLIT == 1 ? 16 : 12)>(part_o, part_lse, out, out_stride, comb, kvh, nh, nkv, lane);
+        merge_parts<(KSPLIT == 1 ? 16 : 12)>(part_o, part_lse, out, out_stride, comb, kvh, nh, nkv, lane, sinks);
       }
     }
   }
@@ -552,7 +575,7 @@ constexpr int kCombineParts = 128;   // parts whose weights fit in LDS at once; 
 __global__ void __launch_bounds__(256)
 attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_lse,
                          uint16_t* __restrict__ out, int out_stride, const Task* __restrict__ tasks, int nh,
-                         int nkv) {
+                         int nkv, const float* __restrict__ sinks) {
   __shared__ float wts[kCombineParts][32];
   __shared__ float row_max[32];
   const Task task = tasks[blockIdx.x];
@@ -574,6 +597,9 @@ attention_combine_kernel(const float* __restrict__ part_o, const float* __restri
       float m2 = wts[0][tid];
 #pragma unroll
       for (int i = 1; i < 8; ++i) m2 = fmaxf(m2, wts[i][tid]);
+      // a row's sink takes part in the maximum, so that its weight below cannot overflow
+      const int hq_row = (task.row0 + tid) / task.qt;
+      if (sinks != nullptr && hq_row < nh / nkv) m2 = fmaxf(m2, sinks[blockIdx.y * (nh / nkv) + hq_row] * kLog2e);
       row_max[tid] = m2;
     }
     __syncthreads();
@@ -624,8 +650,9 @@ attention_combine_kernel(const float* __restrict__ part_o, const float* __restri
     const int r = task.row0 + c;
     const int hq = r / task.qt, tok = task.tok0 + r % task.qt;
     if (idx >= 32 * HD || hq >= g || tok >= count) continue;
+    const float sink_w = sinks != nullptr ? __builtin_amdgcn_exp2f(sinks[kvh * g + hq] * kLog2e - row_max[c]) : 0.f;
     out[(size_t)(tok_base + tok) * out_stride + (size_t)(kvh * g + hq) * HD + d] =
-        f32_to_bf16_bits(acc[it] / wsum[it]);
+        f32_to_bf16_bits(acc[it] / (wsum[it] + sink_w));
   }
 }
 
@@ -671,7 +698,7 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
                                     int out_stride, float* part_o, float* part_lse, const int32_t* tasks, int n_tasks,
                                     int n_combine, const int32_t* block_tables, int max_blocks, float scale,
                                     int window, int nh, int nkv, int ksplit, int row_tiles, int32_t* counters,
-                                    hipStream_t stream) {
+                                    const float* sinks, hipStream_t stream) {
   if (n_tasks <= 0) return 0;
   // row_tiles: 1, or 2: the tasks that write the output cover 64 rows (Task::tiles says so), two waves a task
   if (row_tiles != 1 && !(row_tiles == 2 && kTwoPieces && ksplit == 2)) return ATOMA_ERR_SHAPE;
@@ -689,7 +716,7 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
                        dim3(64 * T * KS), BYTES,                                                                   \
                        stream, t, n_tasks, nkv, (const uint16_t*)q, q_stride, nh, block_tables, max_blocks,        \
                        window, (const uint16_t*)kcache, (const uint16_t*)vcache, (uint16_t*)out, out_stride,       \
-                       part_o, part_lse, scale, counters);                                                         \
+                       part_o, part_lse, scale, counters, sinks);                                                  \
   } while (0)
   if (ksplit == 1) ATOMA_ATTN(4, 1, 0);
   else if (ksplit == 2 && row_tiles == 2) ATOMA_ATTN(4, 2, 2 * kMerge2Bytes, (kTwoPieces ? 2 : 1));
@@ -701,7 +728,7 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
   ATOMA_LAUNCH_CHECK();
   if (n_combine > 0 && counters == nullptr) {
     hipLaunchKernelGGL(attention_combine_kernel, dim3(n_combine, nkv), dim3(256), 0, stream, part_o, part_lse,
-                       (uint16_t*)out, out_stride, t + n_tasks, nh, nkv);
+                       (uint16_t*)out, out_stride, t + n_tasks, nh, nkv, sinks);
     ATOMA_LAUNCH_CHECK();
   }
   return 0;

@@ -1,5 +1,8 @@
 """bfloat16 attention over the paged cache on the matrix cores: task lists on the host, kernels per head size.
 
+The mask is one integer everywhere here (``window``): w > 0 a window of the last w keys, -c < 0 chunks of c
+positions (a token sees the keys of its own chunk up to itself), 0 all keys; ``first_key`` states it.
+
 ``try_attention`` runs ``attention_mfma.hip`` (compiled for the model's head size and the cache's page size on
 first use) when the cache's pages hold a multiple of 16 tokens; otherwise it returns False and the caller runs the
 general kernel.
@@ -217,12 +220,23 @@ def _live_pieces(rows: int, qt: int, live_tokens: int, piece: int = 32):
     return out
 
 
+def first_key(pos, window: int):
+    """The first key that the token at ``pos`` (an integer or an array of them) sees under the mask ``window``:
+    w > 0: the last w keys, its own included; -c < 0: the keys of its own chunk of c positions, counted from the
+    request's first; 0: all keys."""
+    if window > 0:
+        return np.maximum(0, pos - window + 1)
+    if window < 0:
+        return (pos // -window) * -window
+    return pos * 0
+
+
 def _chunk_slots(bucket_keys: int, chunk: int, window: int) -> int:
     """Partial results that a decoded token of a graph's bucket owns: one per chunk of the bucket's keys, or, with
     a window, per chunk that a window can touch wherever it lies (its first chunk is then slot 0)."""
     slots = -(-bucket_keys // chunk)
-    if window > 0:
-        slots = min(slots, -(-window // chunk) + 1)
+    if window != 0:
+        slots = min(slots, -(-abs(window) // chunk) + 1)
     return slots
 
 
@@ -240,7 +254,7 @@ def _tile_tasks(e: int, start: int, count: int, tok_base: int, group: int, windo
     tok0 = np.arange(0, count, qt, dtype=np.int64)                           # [tiles]
     last = np.minimum(tok0 + qt, count)
     k_end = start + last
-    lo = np.maximum(0, start + tok0 - window + 1) if window > 0 else np.zeros_like(tok0)
+    lo = first_key(start + tok0, window)
     kb = (lo // 32) * 32
     tiles = len(tok0)
     t = np.empty((tiles, fours * 4, 12), dtype=np.int32)
@@ -321,16 +335,16 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     n_part = 0
 
     def splits(e):
-        first_key = max(0, int(starts[e]) - window + 1) if window > 0 else 0
+        first = int(first_key(int(starts[e]), window))
         return bucket is not None or (int(counts[e]) <= SPLIT_MAX_TOKENS
-                                      and int(starts[e]) + int(counts[e]) - first_key >= SPLIT_MIN_KEYS)
+                                      and int(starts[e]) + int(counts[e]) - first >= SPLIT_MIN_KEYS)
 
     split_entries = [e for e in range(len(starts)) if splits(e)]
     chunk, waves, merge = CHUNK, 1, False
     if split_entries:
         most = bucket if bucket is not None else max(int(starts[e]) + int(counts[e]) for e in split_entries)
-        if bucket is not None and window > 0:
-            most = min(most, window + CHUNK)
+        if bucket is not None and window != 0:
+            most = min(most, abs(window) + CHUNK)
         chunk, waves = chunk_for(len(split_entries), most, kv_heads)
         waves = min(waves, max_waves)
         merge = merges_in_kernel(most)
@@ -347,7 +361,7 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
         for tok0 in range(0, count, qt):
             last = min(tok0 + qt, count)
             k_end = start + last
-            lo = max(0, start + tok0 - window + 1) if window > 0 else 0
+            lo = int(first_key(start + tok0, window))
             # pieces of the tile that hold at least one live row (the last tile of an entry may be short): 32 rows
             # each for tasks that leave partial results, 32 * row_tiles for those that write the output
             live = _live_pieces(rows, qt, min(qt, count - tok0), 32 if do_split else piece)
@@ -406,10 +420,10 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     s = len(starts)
     starts = starts.astype(np.int64)
     k_end = starts + 1
-    lo = np.maximum(0, starts - window + 1) if window > 0 else np.zeros(s, dtype=np.int64)
+    lo = first_key(starts, window)
     row_chunks = -(-group // 32)
     # the bucket, not the step's longest request, decides between whole ranges and chunks: a graph holds one of them
-    keys = bucket if window <= 0 else min(bucket, window + CHUNK)      # what a token can see
+    keys = bucket if window == 0 else min(bucket, abs(window) + CHUNK)      # what a token can see
     chunk, waves = chunk_for(s, keys, kv_heads, whole_ok=max_waves >= 8, head_size=head_size)
     waves = min(waves, max_waves)
     if chunk == 0:
@@ -490,8 +504,8 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
     page = cache.page_size
     if not page_ok(page) or hd % 16 or not 16 <= hd <= 256:
         return False
-    if window < 0 or sinks is not None:
-        return False
+    if sinks is not None and not (sinks.dtype is torch.float32 and sinks.is_contiguous() and sinks.numel() == nh):
+        raise ValueError("sinks must be contiguous float32, one per query head")
     if q.stride(0) % 8 or q.data_ptr() % 16 or out.stride(0) % 4:
         return False
     if tuple(k_cache.shape[1:]) != (nkv, page * hd) or tuple(v_cache.shape[1:]) != (nkv, page * hd):
@@ -523,6 +537,6 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
     _check(lib(hd, page=page).atoma_attention_mfma(_p(q), q.stride(0), _p(k_cache), _p(v_cache), _p(out), out.stride(0),
                                         _p(part_o), _p(part_lse), _p(tasks), n_main, n_comb, _p(bt), bt.shape[1],
                                         ctypes.c_float(scale), int(window), nh, nkv, ksplit, row_tiles, _p(counters),
-                                        _stream()),
+                                        _p(sinks), _stream()),
            "attention_mfma")
     return True

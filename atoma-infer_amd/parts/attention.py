@@ -103,7 +103,7 @@ class PagedAttention(Mixer):
         kernels, built once per step on the host and shipped with the step's metadata.  ``bucket_tokens`` is None, or
         for a step that only decodes the context length its plan must serve (a multiple of the runner's bucket)."""
         from ..kernels import attention_bf16
-        if self.slopes is not None or self.chunk or self.sinks is not None:
+        if self.slopes is not None:
             return None          # scores with a bias take the general kernel, which needs no plan
         if cache_dtype is torch.bfloat16 and self.hd % 16:
             import warnings
