@@ -142,6 +142,157 @@ expert_gemm_kernel(const TA* __restrict__ a, int lda, int a_div, const float* __
   }
 }
 
+// ---- bfloat16 on the matrix cores -------------------------------------------------------------------------------
+//
+//   gather_scale      xs[place] = bfloat16(score[slot] * x[token of slot]) for every place of perm: the inputs of the
+//                     first product, ordered by expert, so that a tile's rows are contiguous;
+//   expert_gemm_mfma  a workgroup takes a tile of up to 64 places of one expert against 128 rows of that expert's
+//                     weight, v_mfma_f32_16x16x32_bf16 with float32 sums: the weight's fragments come straight from
+//                     global memory (an element is used by one wave only), the tile of activations passes LDS, 64
+//                     columns of K at a time, and is shared by the four waves.  With few places an expert (decode
+//                     steps) the blocks of 16 places without a live one are skipped and the product streams the
+//                     weight once.  SWIGLU: the weight's rows come in blocks of 16 gate rows followed by the 16 up
+//                     rows of the same outputs, a lane then holds a gate value and its up value, and silu(gate) * up
+//                     leaves as bfloat16 [places, ff]; else the float32 result goes to the plane and row of the
+//                     place's slot (choice c of token t: row c * T + t).
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+__global__ void __launch_bounds__(256)
+gather_scale_kernel(const uint16_t* __restrict__ x, int ldx, const float* __restrict__ score,
+                    const int32_t* __restrict__ perm, uint16_t* __restrict__ xs, int K, int top) {
+  const int place = blockIdx.x, slot = perm[place];
+  const float sc = score[slot];
+  const uint16_t* src = x + (size_t)(slot / top) * ldx;
+  for (int k = threadIdx.x; k < K; k += 256) xs[(size_t)place * K + k] = f32_to_bf16_bits(bf16_bits_to_f32(src[k]) * sc);
+}
+
+constexpr int kLdsRow = 64 + 8;     // bfloat16 elements a row of the activations' tile takes in LDS (padded)
+
+template <bool SWIGLU>
+__global__ void __launch_bounds__(256)
+expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, void* __restrict__ c, int ldc,
+                        int N, int K, const int32_t* __restrict__ perm, const int32_t* __restrict__ offsets,
+                        const int32_t* __restrict__ tiles, int top, int plane_rows) {
+  __shared__ __attribute__((aligned(16))) uint16_t at[64 * kLdsRow];
+  const int e = tiles[2 * blockIdx.y];
+  if (e < 0) return;
+  const int row0 = tiles[2 * blockIdx.y + 1];
+  const int rows = min(64, offsets[e + 1] - row0);
+  const int msub = (rows + 15) >> 4;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int n_base = blockIdx.x * 128 + wave * 32;
+  // (a wave whose columns lie beyond N still joins the barriers below; its rows are clamped and never stored)
+  const uint16_t* we = w + (size_t)e * N * K;
+  const uint16_t* wp[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    int n = n_base + s * 16 + r16;
+    if (n > N - 1) n = N - 1;
+    wp[s] = we + (size_t)n * K + kg * 8;
+  }
+  f32x4 acc[2][4];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int m = 0; m < 4; ++m) acc[s][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    bf16x8 wf[2][2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        // (K is a multiple of 32: the last step may have its first half only)
+        if (k0 + kk * 32 < K) wf[kk][s] = *reinterpret_cast<const bf16x8*>(wp[s] + k0 + kk * 32);
+        else wf[kk][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    __syncthreads();          // the tile of the step before has been read
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int idx = tid + i * 256, r = idx >> 3, seg = idx & 7;
+      if (r < msub * 16) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (r < rows && k0 + seg * 8 < K) v = *reinterpret_cast<const uint4*>(a + (size_t)(row0 + r) * K + k0 + seg * 8);
+        *reinterpret_cast<uint4*>(at + r * kLdsRow + seg * 8) = v;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        if (m < msub) {
+          const bf16x8 af = *reinterpret_cast<const bf16x8*>(at + (m * 16 + r16) * kLdsRow + kk * 32 + kg * 8);
+#pragma unroll
+          for (int s = 0; s < 2; ++s)
+            acc[s][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[kk][s], af, acc[s][m], 0, 0, 0);
+        }
+      }
+    }
+  }
+  // lane: place m * 16 + r16 of the tile, columns kg * 4 .. + 3 of each of its two blocks of 16 rows of the weight
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    const int r = m * 16 + r16;
+    if (m >= msub || r >= rows) continue;
+    const int place = row0 + r;
+    if constexpr (SWIGLU) {
+      const int n0 = n_base / 2 + kg * 4;      // outputs: one for every pair of a gate row and an up row
+      uint16_t* dst = (uint16_t*)c + (size_t)place * ldc + n0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (n_base + 16 + kg * 4 + i < N) {
+          const float g = acc[0][m][i];
+          dst[i] = f32_to_bf16_bits(g / (1.0f + expf(-g)) * acc[1][m][i]);
+        }
+      }
+    } else {
+      const int slot = perm[place];
+      const size_t row = plane_rows > 0 ? (size_t)(slot % top) * plane_rows + slot / top : (size_t)place;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const int n0 = n_base + s * 16 + kg * 4;
+        float* dst = (float*)c + row * ldc + n0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n0 + i < N) dst[i] = acc[s][m][i];
+      }
+    }
+  }
+}
+
+extern "C" int atoma_gather_scale(const void* x, int ldx, const float* score, const int32_t* perm, void* xs, int K,
+                                  int top, int n_slots, hipStream_t stream) {
+  if (n_slots <= 0) return 0;
+  if (K <= 0 || ldx < K || top <= 0) return ATOMA_ERR_SHAPE;
+  hipLaunchKernelGGL(gather_scale_kernel, dim3(n_slots), dim3(256), 0, stream, (const uint16_t*)x, ldx, score, perm,
+                     (uint16_t*)xs, K, top);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+// a [places, K] bfloat16 in the order of perm; w [experts, N, K] bfloat16.  swiglu: c bfloat16 [places, N / 2] (ldc),
+// the rows of w in blocks of 16 gate rows and their 16 up rows; else c float32, by place or (plane_rows > 0) by slot
+extern "C" int atoma_expert_gemm_mfma(const void* a, const void* w, void* c, int ldc, int N, int K, const int32_t* perm,
+                                      const int32_t* offsets, const int32_t* tiles, int max_tiles, int top,
+                                      int plane_rows, int swiglu, hipStream_t stream) {
+  if (max_tiles <= 0 || N <= 0) return 0;
+  if (K <= 0 || K % 32 || N % 32 || top <= 0 || max_tiles > 65535 || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) ||
+      ldc < (swiglu ? N / 2 : N))
+    return ATOMA_ERR_SHAPE;
+  dim3 grid((N + 127) / 128, max_tiles), block(256);
+  if (swiglu)
+    hipLaunchKernelGGL((expert_gemm_mfma_kernel<true>), grid, block, 0, stream, (const uint16_t*)a, (const uint16_t*)w,
+                       c, ldc, N, K, perm, offsets, tiles, top, plane_rows);
+  else
+    hipLaunchKernelGGL((expert_gemm_mfma_kernel<false>), grid, block, 0, stream, (const uint16_t*)a,
+                       (const uint16_t*)w, c, ldc, N, K, perm, offsets, tiles, top, plane_rows);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
 extern "C" int atoma_route_topk(const float* logits, int ld, int experts, int top, int32_t* ids, float* weights,
                                 int n_tokens, hipStream_t stream) {
   if (n_tokens <= 0) return 0;

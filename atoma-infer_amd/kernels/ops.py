@@ -480,6 +480,43 @@ def expert_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, perm, offse
         n_slots // top if planes else 0, _stream()), "expert_gemm")
 
 
+def gather_scale(x: torch.Tensor, scores: torch.Tensor, perm: torch.Tensor, top: int) -> torch.Tensor:
+    """xs[place] = bfloat16(scores[slot] * x[slot // top]) for slot = perm[place]: the experts' inputs in their order."""
+    _dev(x, scores, perm)
+    n, k = perm.numel(), x.shape[1]
+    _need(x.dtype is torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1 and x.shape[0] * top == n, "gather_scale: bad x")
+    _f32(scores, "scores", n)
+    _i32(perm, "perm", n)
+    xs = torch.empty((n, k), dtype=torch.bfloat16, device=x.device)
+    _check(_module("experts").atoma_gather_scale(_p(x), x.stride(0) if x.shape[0] > 1 else k, _p(scores), _p(perm),
+                                                 _p(xs), k, int(top), n, _stream()), "gather_scale")
+    return xs
+
+
+def expert_gemm_mfma_ok(n: int, k: int) -> bool:
+    return k % 32 == 0 and n % 32 == 0
+
+
+def expert_gemm_mfma(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, perm, offsets, tiles, top: int, *,
+                     swiglu: bool = False, planes: bool = False) -> None:
+    """The grouped product on the matrix cores: a bfloat16 [places, K] in the order of ``perm``, w bfloat16
+    [experts, N, K].  ``swiglu``: w's rows in blocks of 16 gate rows and their 16 up rows, out bfloat16
+    [places, N / 2] = silu(gate) * up; else out float32 [places, N] or, with ``planes``, [top, T, N] by slot."""
+    _dev(a, w, out, perm, offsets, tiles)
+    n_slots = perm.numel()
+    e, n, k = w.shape
+    _need(a.dtype is torch.bfloat16 and w.dtype is torch.bfloat16 and a.is_contiguous() and w.is_contiguous()
+          and tuple(a.shape) == (n_slots, k) and expert_gemm_mfma_ok(n, k), "expert_gemm_mfma: operands do not fit")
+    cols = n // 2 if swiglu else n
+    _need(out.is_contiguous() and out.numel() == n_slots * cols and out.shape[-1] == cols
+          and out.dtype is (torch.bfloat16 if swiglu else torch.float32) and not (swiglu and planes),
+          "expert_gemm_mfma: bad out")
+    _need(offsets.numel() == e + 1 and tiles.dim() == 2 and tiles.shape[1] == 2, "expert_gemm_mfma: bad grouping")
+    _check(_module("experts").atoma_expert_gemm_mfma(
+        _p(a), _p(w), _p(out), cols, n, k, _p(perm), _p(offsets), _p(tiles), tiles.shape[0], int(top),
+        n_slots // top if planes else 0, 1 if swiglu else 0, _stream()), "expert_gemm_mfma")
+
+
 SPLIT_MAX_VOCAB = 262144       # the largest vocabulary whose rows ``sample_packed(split=True)`` cuts into parts
 
 

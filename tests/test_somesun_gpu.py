@@ -141,7 +141,7 @@ def test_a_far_token_stays_in_the_recurrent_state():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("experts, top, ff", [(4, 2, 48), (3, 1, 64), (5, 5, 24), (70, 3, 16)])
+@pytest.mark.parametrize("experts, top, ff", [(4, 2, 48), (3, 1, 64), (5, 5, 24), (70, 3, 16), (6, 2, 96), (40, 4, 32)])
 def test_routed_experts_alone(experts, top, ff, dtype):
     from atoma_infer_amd.parts import RoutedExperts
     from atoma_infer_amd.weights.random_init import random_tensor
@@ -152,6 +152,9 @@ def test_routed_experts_alone(experts, top, ff, dtype):
         if n != "router":
             w[n] = (w[n] * 10).to(torch.bfloat16).float()
     _load(part, w, dtype)
+    # (the matrix-core products take expert widths that are multiples of 32 in bfloat16; the others, and the 32-bit
+    # path, run float32 multiply-adds)
+    assert part.mfma == (dtype is torch.bfloat16 and ff % 32 == 0)
     g = torch.Generator().manual_seed(experts)
     for t in (1, 3, 150):          # one row tile, and experts whose rows fill more than one
         h = torch.randn(t, width, generator=g).to(torch.bfloat16).float()
