@@ -7,10 +7,11 @@
 //                      inputs before an entry's first token come from the request's state), q and k to unit length per
 //                      head (q also times dim^-1/2), beta = sigmoid(b), g = exp(-exp(A_log) softplus(a + dt_bias));
 //   delta_conv_state   per request: the last taps - 1 inputs of the convolution, for the request's next step;
-//   delta_scan         per (request, head, 8 columns of S): the recurrence over the entry's tokens in order, S read from
+//   delta_scan         per (request, head, 16 columns of S): the recurrence over the entry's tokens in order, S read from
 //                      the request's state slot before and written back after.  A column of S lives in the registers
-//                      of 8 neighbouring lanes (dim / 8 rows each, rounded up), so a token costs a lane a few dozen
-//                      multiply-adds and one three-step exchange among those lanes;
+//                      of 16 neighbouring lanes (dim / 16 rows each, rounded up), so a token costs a lane a few dozen
+//                      multiply-adds and one four-step exchange among those lanes; the tokens' inputs pass LDS in
+//                      blocks, fetched a block ahead;
 //   delta_out          per token and head: o / sqrt(mean(o^2) + eps) * w * sigmoid(gate), in the activation dtype.
 // The order of every sum depends on the sizes alone, so a token's result does not depend on how the request was cut
 // into steps or on what else the step holds.
@@ -34,7 +35,7 @@ __global__ void __launch_bounds__(256)
 delta_prepare_kernel(const float* __restrict__ proj, DeltaShape sh, const int32_t* __restrict__ token_seq,
                      const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
                      const float* __restrict__ state, size_t state_stride, const float* __restrict__ taps_w,
-                     const float* __restrict__ dt_pre, const float* __restrict__ dt_bias,
+                     const float* __restrict__ dt_pre, int ld_dt, const float* __restrict__ dt_bias,
                      const float* __restrict__ a_log, float* __restrict__ qn, float* __restrict__ kn,
                      float* __restrict__ vn, float* __restrict__ beta, float* __restrict__ decay) {
   extern __shared__ float act[];       // the token's channels after convolution and SiLU
@@ -42,6 +43,17 @@ delta_prepare_kernel(const float* __restrict__ proj, DeltaShape sh, const int32_
   const int e = token_seq[t];
   const int n = t - q_start[e];        // the token's index inside its entry
   const int nqk = sh.kv_heads * sh.dim, nv = sh.heads * sh.vdim, channels = 2 * nqk + nv;
+  if (blockIdx.y == 1) {
+    // the token's second workgroup: the gates of the recurrence, which need nothing of the convolution
+    for (int h = threadIdx.x; h < sh.heads; h += 256)
+      beta[(size_t)t * sh.heads + h] = sigmoidf_(proj[(size_t)t * sh.ldp + sh.off_b + h]);
+    const int nd = sh.heads * sh.dim;
+    for (int c = threadIdx.x; c < nd; c += 256) {
+      const float rate = expf(a_log[c / sh.dim]);
+      decay[(size_t)t * nd + c] = expf(-rate * softplusf_(dt_pre[(size_t)t * ld_dt + c] + dt_bias[c]));
+    }
+    return;
+  }
   const float* conv_state = state + (size_t)state_slots[e] * state_stride;
   for (int c = threadIdx.x; c < channels; c += 256) {
     const int col = c < nqk ? sh.off_q + c : c < 2 * nqk ? sh.off_k + (c - nqk) : sh.off_v + (c - 2 * nqk);
@@ -69,13 +81,6 @@ delta_prepare_kernel(const float* __restrict__ proj, DeltaShape sh, const int32_
     for (int i = lane; i < sh.dim; i += 64) dst[i] = x[i] * inv;
   }
   for (int c = threadIdx.x; c < nv; c += 256) vn[(size_t)t * nv + c] = act[2 * nqk + c];
-  for (int h = threadIdx.x; h < sh.heads; h += 256)
-    beta[(size_t)t * sh.heads + h] = sigmoidf_(proj[(size_t)t * sh.ldp + sh.off_b + h]);
-  const int nd = sh.heads * sh.dim;
-  for (int c = threadIdx.x; c < nd; c += 256) {
-    const float rate = expf(a_log[c / sh.dim]);
-    decay[(size_t)t * nd + c] = expf(-rate * softplusf_(dt_pre[(size_t)t * nd + c] + dt_bias[c]));
-  }
 }
 
 // one thread a (entry, channel): the state's rows in ascending order, so that a row is read before it is overwritten
@@ -96,15 +101,34 @@ delta_conv_state_kernel(const float* __restrict__ proj, DeltaShape sh, const int
   }
 }
 
-// R: rows of S a lane holds; 8 lanes share a column, so dim <= 8 R
+// Sum over the 16 lanes of a DPP row; every lane gets the same sum (the pairs of each step add the same two numbers).
+__device__ __forceinline__ float row16_sum(float x) {
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xf, 0xf, false));    // lanes i ^ 1
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xf, 0xf, false));    // lanes i ^ 2
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x141, 0xf, 0xf, false));   // the other quad of 8
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x140, 0xf, 0xf, false));   // the other half of 16
+  return x;
+}
+
+// R: rows of S a lane holds.  16 lanes (a DPP row) share a column of S, so dim <= 16 R; a wave holds 4 columns, a
+// workgroup of four waves 16.  The tokens' q, k, decay (for the head), v (for the 16 columns) and beta pass LDS in
+// blocks of TB tokens: the next block is fetched from memory while this one is worked on, so the walk over the tokens
+// waits for LDS only.
 template <int R>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
 delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vn,
                   const float* __restrict__ beta, const float* __restrict__ decay, DeltaShape sh,
                   const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
                   float* __restrict__ state, size_t state_stride, size_t s_offset, float* __restrict__ o) {
-  const int lane = threadIdx.x;
-  const int col = blockIdx.x * 8 + (lane >> 3), part = lane & 7;
+  constexpr int DP = 16 * R;                   // dim rounded up; rows beyond dim hold zeros
+  constexpr int TB = R <= 8 ? 16 : 8;          // tokens a block
+  constexpr int PER = TB * DP / 256;           // elements of q (k, decay) a thread fetches a block
+  __shared__ float sq[2][TB][DP], sk[2][TB][DP], sg[2][TB][DP];
+  __shared__ float sv[2][TB][16], sb[2][TB];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int part = lane & 15;
+  const int col_local = wave * 4 + (lane >> 4);
+  const int col = blockIdx.x * 16 + col_local;
   const int h = blockIdx.y, e = blockIdx.z;
   const int kv = h / (sh.heads / sh.kv_heads);
   const int dim = sh.dim, vdim = sh.vdim;
@@ -118,48 +142,70 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, co
   for (int r = 0; r < R; ++r) s[r] = (col_ok && i0 + r < dim) ? sp[r] : 0.f;
 
   const int nqk = sh.kv_heads * dim, nd = sh.heads * dim, nv = sh.heads * vdim;
-  struct Tok {
-    float q[R], k[R], g[R], v, b;
+  float pq[PER], pk[PER], pg[PER], pv = 0.f, pb = 0.f;
+  // block b's share of this thread: element idx = tid + j * 256 of [TB][DP]; v: thread tid of [TB][16]; beta: tid < TB
+  auto fetch = [&](int b) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int idx = tid + j * 256, tok = idx / DP, i = idx % DP;
+      const int n = b * TB + tok;
+      const bool ok = n < count && i < dim;
+      const size_t t = (size_t)(first + n);
+      pq[j] = ok ? qn[t * nqk + (size_t)kv * dim + i] : 0.f;
+      pk[j] = ok ? kn[t * nqk + (size_t)kv * dim + i] : 0.f;
+      pg[j] = ok ? decay[t * nd + (size_t)h * dim + i] : 0.f;
+    }
+    if (tid < TB * 16) {
+      const int tok = tid >> 4, c = blockIdx.x * 16 + (tid & 15);
+      const int n = b * TB + tok;
+      pv = (n < count && c < vdim) ? vn[(size_t)(first + n) * nv + (size_t)h * vdim + c] : 0.f;
+    }
+    if (tid < TB) pb = (b * TB + tid < count) ? beta[(size_t)(first + b * TB + tid) * sh.heads + h] : 0.f;
   };
-  auto load = [&](Tok& x, int n) {
-    const size_t t = (size_t)(first + n);
-    const float* qp = qn + t * nqk + (size_t)kv * dim + i0;
-    const float* kp = kn + t * nqk + (size_t)kv * dim + i0;
-    const float* gp = decay + t * nd + (size_t)h * dim + i0;
+  auto stash = [&](int buf) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const bool ok = i0 + r < dim;
-      x.q[r] = ok ? qp[r] : 0.f;
-      x.k[r] = ok ? kp[r] : 0.f;
-      x.g[r] = ok ? gp[r] : 0.f;
+    for (int j = 0; j < PER; ++j) {
+      const int idx = tid + j * 256, tok = idx / DP, i = idx % DP;
+      sq[buf][tok][i] = pq[j];
+      sk[buf][tok][i] = pk[j];
+      sg[buf][tok][i] = pg[j];
     }
-    x.v = col_ok ? vn[t * nv + (size_t)h * vdim + col] : 0.f;
-    x.b = beta[t * sh.heads + h];
+    if (tid < TB * 16) sv[buf][tid >> 4][tid & 15] = pv;
+    if (tid < TB) sb[buf][tid] = pb;
   };
-  Tok cur, nxt;
-  if (count > 0) load(cur, 0);
-  for (int n = 0; n < count; ++n) {
-    if (n + 1 < count) load(nxt, n + 1);
-    float d1 = 0.f, d2 = 0.f, kq = 0.f;
+  const int blocks = (count + TB - 1) / TB;
+  if (blocks > 0) {
+    fetch(0);
+    stash(0);
+  }
+  __syncthreads();
+  for (int b = 0; b < blocks; ++b) {
+    const int buf = b & 1;
+    if (b + 1 < blocks) fetch(b + 1);
+    const int n_tok = min(TB, count - b * TB);
+    for (int tok = 0; tok < n_tok; ++tok) {
+      float d1 = 0.f, d2 = 0.f, kq = 0.f;
+      float kr[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      s[r] *= cur.g[r];
-      d1 = fmaf(s[r], cur.k[r], d1);
-      d2 = fmaf(s[r], cur.q[r], d2);
-      kq = fmaf(cur.k[r], cur.q[r], kq);
+      for (int r = 0; r < R; ++r) {
+        const float g = sg[buf][tok][i0 + r], q = sq[buf][tok][i0 + r];
+        kr[r] = sk[buf][tok][i0 + r];
+        s[r] *= g;
+        d1 = fmaf(s[r], kr[r], d1);
+        d2 = fmaf(s[r], q, d2);
+        kq = fmaf(kr[r], q, kq);
+      }
+      d1 = row16_sum(d1);
+      d2 = row16_sum(d2);
+      kq = row16_sum(kq);
+      const float u = sb[buf][tok] * (sv[buf][tok][col_local] - d1);
+      // o = S_new^T q with S_new = diag(g) S + k u^T
+      if (part == 0 && col_ok) o[(size_t)(first + b * TB + tok) * nv + (size_t)h * vdim + col] = fmaf(u, kq, d2);
+#pragma unroll
+      for (int r = 0; r < R; ++r) s[r] = fmaf(kr[r], u, s[r]);
     }
-#pragma unroll
-    for (int off = 1; off < 8; off <<= 1) {
-      d1 += __shfl_xor(d1, off, 64);
-      d2 += __shfl_xor(d2, off, 64);
-      kq += __shfl_xor(kq, off, 64);
-    }
-    const float u = cur.b * (cur.v - d1);
-    // o = S_new^T q with S_new = diag(g) S + k u^T
-    if (part == 0 && col_ok) o[(size_t)(first + n) * nv + (size_t)h * vdim + col] = fmaf(u, kq, d2);
-#pragma unroll
-    for (int r = 0; r < R; ++r) s[r] = fmaf(cur.k[r], u, s[r]);
-    cur = nxt;
+    if (b + 1 < blocks) stash(buf ^ 1);
+    __syncthreads();
   }
   if (col_ok) {
 #pragma unroll
@@ -170,8 +216,8 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, co
 
 template <typename TO>
 __global__ void __launch_bounds__(256)
-delta_out_kernel(const float* __restrict__ o, const float* __restrict__ gate_pre, const float* __restrict__ w,
-                 float eps, TO* __restrict__ out, int heads, int vdim) {
+delta_out_kernel(const float* __restrict__ o, const float* __restrict__ gate_pre, int ld_gate,
+                 const float* __restrict__ w, float eps, TO* __restrict__ out, int heads, int vdim) {
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int h = wave; h < heads; h += 4) {
     const size_t base = ((size_t)t * heads + h) * vdim;
@@ -180,7 +226,8 @@ delta_out_kernel(const float* __restrict__ o, const float* __restrict__ gate_pre
     ss = wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
     for (int j = lane; j < vdim; j += 64)
-      out[base + j] = from_f32<TO>(o[base + j] * inv * w[j] * sigmoidf_(gate_pre[base + j]));
+      out[base + j] = from_f32<TO>(o[base + j] * inv * w[j] *
+                                   sigmoidf_(gate_pre[(size_t)t * ld_gate + (size_t)h * vdim + j]));
   }
 }
 
@@ -192,16 +239,18 @@ static bool shape_ok(const DeltaShape& sh) {
 extern "C" int atoma_delta_prepare(const float* proj, int ldp, int off_q, int off_k, int off_v, int off_b, int heads,
                                    int kv_heads, int dim, int vdim, int taps, const int32_t* token_seq,
                                    const int32_t* q_start, const int32_t* state_slots, float* state,
-                                   size_t state_stride, const float* taps_w, const float* dt_pre, const float* dt_bias,
+                                   size_t state_stride, const float* taps_w, const float* dt_pre, int ld_dt,
+                                   const float* dt_bias,
                                    const float* a_log, float* qn, float* kn, float* vn, float* beta, float* decay,
                                    int n_tokens, int n_entries, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   DeltaShape sh{heads, kv_heads, dim, vdim, taps, ldp, off_q, off_k, off_v, off_b};
   if (!shape_ok(sh) || n_entries <= 0 || n_entries > 65535) return ATOMA_ERR_SHAPE;
+  // (a token has two workgroups: convolution, SiLU and unit lengths; beta and decay)
   const int channels = 2 * kv_heads * dim + heads * vdim;
   if ((size_t)channels * sizeof(float) > 60 * 1024) return ATOMA_ERR_SHAPE;
-  hipLaunchKernelGGL(delta_prepare_kernel, dim3(n_tokens), dim3(256), channels * sizeof(float), stream, proj, sh,
-                     token_seq, q_start, state_slots, state, state_stride, taps_w, dt_pre, dt_bias, a_log, qn, kn, vn,
+  hipLaunchKernelGGL(delta_prepare_kernel, dim3(n_tokens, 2), dim3(256), channels * sizeof(float), stream, proj, sh,
+                     token_seq, q_start, state_slots, state, state_stride, taps_w, dt_pre, ld_dt, dt_bias, a_log, qn, kn, vn,
                      beta, decay);
   ATOMA_LAUNCH_CHECK();
   if (taps > 1) {
@@ -220,30 +269,30 @@ extern "C" int atoma_delta_scan(const float* qn, const float* kn, const float* v
   DeltaShape sh{heads, kv_heads, dim, vdim, taps, 1, 0, 0, 0, 0};
   if (!shape_ok(sh) || n_entries > 65535 || heads > 65535) return ATOMA_ERR_SHAPE;
   const size_t s_offset = (size_t)(taps - 1) * (2 * kv_heads * dim + heads * vdim);
-  dim3 grid((vdim + 7) / 8, heads, n_entries), block(64);
+  dim3 grid((vdim + 15) / 16, heads, n_entries), block(256);
 #define ATOMA_SCAN(R_)                                                                                            \
   hipLaunchKernelGGL((delta_scan_kernel<R_>), grid, block, 0, stream, qn, kn, vn, beta, decay, sh, q_start,       \
                      state_slots, state, state_stride, s_offset, o)
-  if (dim <= 16) ATOMA_SCAN(2);
-  else if (dim <= 32) ATOMA_SCAN(4);
-  else if (dim <= 64) ATOMA_SCAN(8);
-  else if (dim <= 128) ATOMA_SCAN(16);
-  else ATOMA_SCAN(32);
+  if (dim <= 16) ATOMA_SCAN(1);
+  else if (dim <= 32) ATOMA_SCAN(2);
+  else if (dim <= 64) ATOMA_SCAN(4);
+  else if (dim <= 128) ATOMA_SCAN(8);
+  else ATOMA_SCAN(16);
 #undef ATOMA_SCAN
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
 
-extern "C" int atoma_delta_out(const float* o, const float* gate_pre, const float* w, float eps, void* out,
+extern "C" int atoma_delta_out(const float* o, const float* gate_pre, int ld_gate, const float* w, float eps, void* out,
                                int out_dtype, int n_tokens, int heads, int vdim, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
-  if (heads <= 0 || vdim <= 0) return ATOMA_ERR_SHAPE;
+  if (heads <= 0 || vdim <= 0 || ld_gate < heads * vdim) return ATOMA_ERR_SHAPE;
   if (out_dtype == kF32)
-    hipLaunchKernelGGL((delta_out_kernel<float>), dim3(n_tokens), dim3(256), 0, stream, o, gate_pre, w, eps,
-                       (float*)out, heads, vdim);
+    hipLaunchKernelGGL((delta_out_kernel<float>), dim3(n_tokens), dim3(256), 0, stream, o, gate_pre, ld_gate, w,
+                       eps, (float*)out, heads, vdim);
   else if (out_dtype == kBF16)
-    hipLaunchKernelGGL((delta_out_kernel<bf16_t>), dim3(n_tokens), dim3(256), 0, stream, o, gate_pre, w, eps,
-                       (bf16_t*)out, heads, vdim);
+    hipLaunchKernelGGL((delta_out_kernel<bf16_t>), dim3(n_tokens), dim3(256), 0, stream, o, gate_pre, ld_gate, w,
+                       eps, (bf16_t*)out, heads, vdim);
   else
     return ATOMA_ERR_DTYPE;
   ATOMA_LAUNCH_CHECK();

@@ -56,7 +56,7 @@ route_topk_kernel(const float* __restrict__ logits, int ld, int experts, int top
 
 __global__ void __launch_bounds__(1024)
 route_group_kernel(const int32_t* __restrict__ ids, int n_slots, int experts, int32_t* __restrict__ perm,
-                   int32_t* __restrict__ offsets, int32_t* __restrict__ tiles, int max_tiles) {
+                   int32_t* __restrict__ offsets, int32_t* __restrict__ tiles, int max_tiles, int tile_m) {
   __shared__ int32_t counts[1024];
   __shared__ int32_t cursor[1024];
   for (int e = threadIdx.x; e < experts; e += 1024) counts[e] = 0;
@@ -68,7 +68,7 @@ route_group_kernel(const int32_t* __restrict__ ids, int n_slots, int experts, in
     for (int e = 0; e < experts; ++e) {
       offsets[e] = at;
       cursor[e] = at;
-      for (int r = 0; r < counts[e]; r += kTileM) {
+      for (int r = 0; r < counts[e]; r += tile_m) {
         tiles[2 * n] = e;
         tiles[2 * n + 1] = at + r;
         ++n;
@@ -149,7 +149,8 @@ expert_gemm_kernel(const TA* __restrict__ a, int lda, int a_div, const float* __
 //   expert_gemm_mfma  a workgroup takes a tile of up to 64 places of one expert against 128 rows of that expert's
 //                     weight, v_mfma_f32_16x16x32_bf16 with float32 sums: the weight's fragments come straight from
 //                     global memory (an element is used by one wave only), the tile of activations passes LDS, 64
-//                     columns of K at a time, and is shared by the four waves.  With few places an expert (decode
+//                     columns of K at a time, and is shared by the four waves; both are asked for a step ahead.  Tiles
+//                     hold 64 places, or 128 where the experts have many (prompts).  With few places an expert (decode
 //                     steps) the blocks of 16 places without a live one are skipped and the product streams the
 //                     weight once.  SWIGLU: the weight's rows come in blocks of 16 gate rows followed by the 16 up
 //                     rows of the same outputs, a lane then holds a gate value and its up value, and silu(gate) * up
@@ -169,16 +170,18 @@ gather_scale_kernel(const uint16_t* __restrict__ x, int ldx, const float* __rest
 
 constexpr int kLdsRow = 64 + 8;     // bfloat16 elements a row of the activations' tile takes in LDS (padded)
 
-template <bool SWIGLU>
+template <bool SWIGLU, int TM>
 __global__ void __launch_bounds__(256)
 expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, void* __restrict__ c, int ldc,
                         int N, int K, const int32_t* __restrict__ perm, const int32_t* __restrict__ offsets,
                         const int32_t* __restrict__ tiles, int top, int plane_rows) {
-  __shared__ __attribute__((aligned(16))) uint16_t at[64 * kLdsRow];
+  constexpr int MS = TM / 16;          // blocks of 16 places a tile
+  constexpr int AP = TM / 32;          // 16-byte pieces of the activations' tile a thread moves a step
+  __shared__ __attribute__((aligned(16))) uint16_t at[TM * kLdsRow];
   const int e = tiles[2 * blockIdx.y];
   if (e < 0) return;
   const int row0 = tiles[2 * blockIdx.y + 1];
-  const int rows = min(64, offsets[e + 1] - row0);
+  const int rows = min(TM, offsets[e + 1] - row0);
   const int msub = (rows + 15) >> 4;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
@@ -192,37 +195,46 @@ expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restri
     if (n > N - 1) n = N - 1;
     wp[s] = we + (size_t)n * K + kg * 8;
   }
-  f32x4 acc[2][4];
+  f32x4 acc[2][MS];
 #pragma unroll
   for (int s = 0; s < 2; ++s)
 #pragma unroll
-    for (int m = 0; m < 4; ++m) acc[s][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int m = 0; m < MS; ++m) acc[s][m] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int k0 = 0; k0 < K; k0 += 64) {
-    bf16x8 wf[2][2];
+  // The operands of a step are asked for a step ahead: the weight's fragments wait in registers, the activations' pieces
+  // too, until the tile of the step before has been read and they may go to LDS.
+  bf16x8 wf[2][2], wn[2][2];
+  uint4 ar[AP];
+  auto fetch = [&](int k0, bf16x8 (&dst)[2][2]) {
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         // (K is a multiple of 32: the last step may have its first half only)
-        if (k0 + kk * 32 < K) wf[kk][s] = *reinterpret_cast<const bf16x8*>(wp[s] + k0 + kk * 32);
-        else wf[kk][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (k0 + kk * 32 < K) dst[kk][s] = *reinterpret_cast<const bf16x8*>(wp[s] + k0 + kk * 32);
+        else dst[kk][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
       }
+#pragma unroll
+    for (int i = 0; i < AP; ++i) {
+      const int idx = tid + i * 256, r = idx >> 3, seg = idx & 7;
+      ar[i] = make_uint4(0, 0, 0, 0);
+      if (r < rows && k0 + seg * 8 < K) ar[i] = *reinterpret_cast<const uint4*>(a + (size_t)(row0 + r) * K + k0 + seg * 8);
+    }
+  };
+  fetch(0, wf);
+  for (int k0 = 0; k0 < K; k0 += 64) {
     __syncthreads();          // the tile of the step before has been read
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < AP; ++i) {
       const int idx = tid + i * 256, r = idx >> 3, seg = idx & 7;
-      if (r < msub * 16) {
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (r < rows && k0 + seg * 8 < K) v = *reinterpret_cast<const uint4*>(a + (size_t)(row0 + r) * K + k0 + seg * 8);
-        *reinterpret_cast<uint4*>(at + r * kLdsRow + seg * 8) = v;
-      }
+      if (r < msub * 16) *reinterpret_cast<uint4*>(at + r * kLdsRow + seg * 8) = ar[i];
     }
     __syncthreads();
+    if (k0 + 64 < K) fetch(k0 + 64, wn);
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
+      for (int m = 0; m < MS; ++m) {
         if (m < msub) {
           const bf16x8 af = *reinterpret_cast<const bf16x8*>(at + (m * 16 + r16) * kLdsRow + kk * 32 + kg * 8);
 #pragma unroll
@@ -231,10 +243,14 @@ expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restri
         }
       }
     }
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) wf[kk][s] = wn[kk][s];
   }
   // lane: place m * 16 + r16 of the tile, columns kg * 4 .. + 3 of each of its two blocks of 16 rows of the weight
 #pragma unroll
-  for (int m = 0; m < 4; ++m) {
+  for (int m = 0; m < MS; ++m) {
     const int r = m * 16 + r16;
     if (m >= msub || r >= rows) continue;
     const int place = row0 + r;
@@ -277,18 +293,20 @@ extern "C" int atoma_gather_scale(const void* x, int ldx, const float* score, co
 // the rows of w in blocks of 16 gate rows and their 16 up rows; else c float32, by place or (plane_rows > 0) by slot
 extern "C" int atoma_expert_gemm_mfma(const void* a, const void* w, void* c, int ldc, int N, int K, const int32_t* perm,
                                       const int32_t* offsets, const int32_t* tiles, int max_tiles, int top,
-                                      int plane_rows, int swiglu, hipStream_t stream) {
+                                      int plane_rows, int swiglu, int tile_m, hipStream_t stream) {
   if (max_tiles <= 0 || N <= 0) return 0;
-  if (K <= 0 || K % 32 || N % 32 || top <= 0 || max_tiles > 65535 || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) ||
+  if (K <= 0 || K % 32 || N % 32 || (tile_m != 64 && tile_m != 128) || top <= 0 || max_tiles > 65535 || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) ||
       ldc < (swiglu ? N / 2 : N))
     return ATOMA_ERR_SHAPE;
   dim3 grid((N + 127) / 128, max_tiles), block(256);
-  if (swiglu)
-    hipLaunchKernelGGL((expert_gemm_mfma_kernel<true>), grid, block, 0, stream, (const uint16_t*)a, (const uint16_t*)w,
-                       c, ldc, N, K, perm, offsets, tiles, top, plane_rows);
-  else
-    hipLaunchKernelGGL((expert_gemm_mfma_kernel<false>), grid, block, 0, stream, (const uint16_t*)a,
-                       (const uint16_t*)w, c, ldc, N, K, perm, offsets, tiles, top, plane_rows);
+#define ATOMA_EGM(SW, TM_)                                                                                       \
+  hipLaunchKernelGGL((expert_gemm_mfma_kernel<SW, TM_>), grid, block, 0, stream, (const uint16_t*)a,             \
+                     (const uint16_t*)w, c, ldc, N, K, perm, offsets, tiles, top, plane_rows)
+  if (swiglu && tile_m == 64) ATOMA_EGM(true, 64);
+  else if (swiglu) ATOMA_EGM(true, 128);
+  else if (tile_m == 64) ATOMA_EGM(false, 64);
+  else ATOMA_EGM(false, 128);
+#undef ATOMA_EGM
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
@@ -303,18 +321,20 @@ extern "C" int atoma_route_topk(const float* logits, int ld, int experts, int to
   return 0;
 }
 
-// the most row tiles that n_slots slots of `experts` experts can need
-extern "C" int atoma_route_max_tiles(int n_slots, int experts) {
-  const int full = n_slots / kTileM + experts;
+// the most row tiles of tile_m places that n_slots slots of `experts` experts can need
+extern "C" int atoma_route_max_tiles(int n_slots, int experts, int tile_m) {
+  const int full = n_slots / tile_m + experts;
   return full < n_slots ? full : (n_slots > 0 ? n_slots : 1);
 }
 
 extern "C" int atoma_route_group(const int32_t* ids, int n_slots, int experts, int32_t* perm, int32_t* offsets,
-                                 int32_t* tiles, int max_tiles, hipStream_t stream) {
+                                 int32_t* tiles, int max_tiles, int tile_m, hipStream_t stream) {
   if (n_slots <= 0) return 0;
-  if (experts <= 0 || experts > 1024 || max_tiles < atoma_route_max_tiles(n_slots, experts)) return ATOMA_ERR_SHAPE;
+  if (experts <= 0 || experts > 1024 || (tile_m != 64 && tile_m != 128) ||
+      max_tiles < atoma_route_max_tiles(n_slots, experts, tile_m))
+    return ATOMA_ERR_SHAPE;
   hipLaunchKernelGGL(route_group_kernel, dim3(1), dim3(1024), 0, stream, ids, n_slots, experts, perm, offsets, tiles,
-                     max_tiles);
+                     max_tiles, tile_m);
   ATOMA_LAUNCH_CHECK();
   return 0;
 }

@@ -61,6 +61,140 @@ add_normed_kernel(float* __restrict__ resid, Term a, Term b, int n_terms, const 
   for (int i = threadIdx.x; i < width; i += 256) out[base + i] = from_f32<TO>(row[i] * inv2 * w_next[i]);
 }
 
+// The same for rows whose width is a multiple of 4, at most 1024 * MAXJ columns, with 16-byte aligned operands: a
+// thread keeps its columns in registers through all three passes, and the loads of a pass (up to four planes of a term
+// at a time) are issued together.
+struct f4 {
+  float v[4];
+};
+
+__device__ __forceinline__ f4 load4(const float* p) {
+  const float4 x = *reinterpret_cast<const float4*>(p);
+  return f4{{x.x, x.y, x.z, x.w}};
+}
+
+__device__ __forceinline__ f4 load4(const bf16_t* p) {
+  const uint2 x = *reinterpret_cast<const uint2*>(p);
+  return f4{{bf16_bits_to_f32((uint16_t)(x.x & 0xffff)), bf16_bits_to_f32((uint16_t)(x.x >> 16)),
+             bf16_bits_to_f32((uint16_t)(x.y & 0xffff)), bf16_bits_to_f32((uint16_t)(x.y >> 16))}};
+}
+
+__device__ __forceinline__ void store4(float* p, const f4& x) {
+  *reinterpret_cast<float4*>(p) = make_float4(x.v[0], x.v[1], x.v[2], x.v[3]);
+}
+
+__device__ __forceinline__ void store4(bf16_t* p, const f4& x) {
+  uint2 o;
+  o.x = (uint32_t)f32_to_bf16_bits(x.v[0]) | ((uint32_t)f32_to_bf16_bits(x.v[1]) << 16);
+  o.y = (uint32_t)f32_to_bf16_bits(x.v[2]) | ((uint32_t)f32_to_bf16_bits(x.v[3]) << 16);
+  *reinterpret_cast<uint2*>(p) = o;
+}
+
+template <typename TD, int MAXJ>
+__device__ __forceinline__ void add_term(f4 (&d)[MAXJ], const Term& t, size_t base, int n4) {
+  const TD* p0 = (const TD*)t.data + base;
+  f4 sum[MAXJ];
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j) sum[j] = f4{{0.f, 0.f, 0.f, 0.f}};
+  for (int s0 = 0; s0 < t.planes; s0 += 4) {
+    f4 x[4][MAXJ];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int s = s0 + q < t.planes ? s0 + q : t.planes - 1;
+#pragma unroll
+      for (int j = 0; j < MAXJ; ++j) {
+        const int c = threadIdx.x + j * 256;
+        if (c < n4) x[q][j] = load4(p0 + s * t.plane_stride + 4 * c);
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      if (s0 + q < t.planes)
+#pragma unroll
+        for (int j = 0; j < MAXJ; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) sum[j].v[i] += x[q][j].v[i];
+  }
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) d[j].v[i] += sum[j].v[i] * t.scale;
+}
+
+template <typename TO, int MAXJ>
+__global__ void __launch_bounds__(256)
+add_normed_vec_kernel(float* __restrict__ resid, Term a, Term b, int n_terms, const float* __restrict__ w_post,
+                      const float* __restrict__ w_next, TO* __restrict__ out, int width, float eps_post,
+                      float eps_next) {
+  __shared__ float scratch[4];
+  const size_t base = (size_t)blockIdx.x * width;
+  const int n4 = width >> 2;
+  f4 d[MAXJ], x[MAXJ];
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j) {
+    d[j] = f4{{0.f, 0.f, 0.f, 0.f}};
+    const int c = threadIdx.x + j * 256;
+    if (c < n4) x[j] = load4(resid + base + 4 * c);
+  }
+  if (a.dtype == kF32) add_term<float, MAXJ>(d, a, base, n4);
+  else add_term<bf16_t, MAXJ>(d, a, base, n4);
+  if (n_terms > 1) {
+    if (b.dtype == kF32) add_term<float, MAXJ>(d, b, base, n4);
+    else add_term<bf16_t, MAXJ>(d, b, base, n4);
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j)
+    if (threadIdx.x + j * 256 < n4)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ss += d[j].v[i] * d[j].v[i];
+  ss = block_sum<4>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps_post);
+  float ss2 = 0.f;
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j) {
+    const int c = threadIdx.x + j * 256;
+    if (c < n4) {
+      const f4 wp = load4(w_post + 4 * c);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        x[j].v[i] += d[j].v[i] * inv * wp.v[i];
+        ss2 += x[j].v[i] * x[j].v[i];
+      }
+      store4(resid + base + 4 * c, x[j]);
+    }
+  }
+  if (out == nullptr) return;
+  ss2 = block_sum<4>(ss2, scratch);
+  const float inv2 = 1.0f / sqrtf(ss2 / (float)width + eps_next);
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j) {
+    const int c = threadIdx.x + j * 256;
+    if (c < n4) {
+      const f4 wn = load4(w_next + 4 * c);
+      f4 y;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) y.v[i] = x[j].v[i] * inv2 * wn.v[i];
+      store4(out + base + 4 * c, y);
+    }
+  }
+}
+
+template <typename TO>
+static void launch_vec(dim3 grid, hipStream_t stream, float* resid, const Term& a, const Term& b, int n_terms,
+                       const float* w_post, const float* w_next, void* out, int width, float eps_post, float eps_next) {
+  const dim3 block(256);
+  if (width <= 2048)
+    hipLaunchKernelGGL((add_normed_vec_kernel<TO, 2>), grid, block, 0, stream, resid, a, b, n_terms, w_post, w_next,
+                       (TO*)out, width, eps_post, eps_next);
+  else if (width <= 4096)
+    hipLaunchKernelGGL((add_normed_vec_kernel<TO, 4>), grid, block, 0, stream, resid, a, b, n_terms, w_post, w_next,
+                       (TO*)out, width, eps_post, eps_next);
+  else
+    hipLaunchKernelGGL((add_normed_vec_kernel<TO, 8>), grid, block, 0, stream, resid, a, b, n_terms, w_post, w_next,
+                       (TO*)out, width, eps_post, eps_next);
+}
+
 // terms: data pointers, dtypes, planes, plane strides and scales of one or two terms, each [planes, n_rows, width]
 extern "C" int atoma_add_normed(float* resid, const void* d0, int dtype0, int planes0, size_t stride0, float scale0,
                                 const void* d1, int dtype1, int planes1, size_t stride1, float scale1,
@@ -73,7 +207,14 @@ extern "C" int atoma_add_normed(float* resid, const void* d0, int dtype0, int pl
   const int n_terms = d1 != nullptr ? 2 : 1;
   const size_t lds = (size_t)width * sizeof(float);
   dim3 grid(n_rows), block(256);
-  if (out == nullptr || out_dtype == kF32)
+  auto aligned = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+  const bool vec = width % 4 == 0 && width <= 8192 && aligned(resid) && aligned(d0) && aligned(d1) && aligned(w_post) &&
+                   aligned(w_next) && aligned(out) && stride0 % 4 == 0 && (d1 == nullptr || stride1 % 4 == 0);
+  if (vec && (out == nullptr || out_dtype == kF32))
+    launch_vec<float>(grid, stream, resid, a, b, n_terms, w_post, w_next, out, width, eps_post, eps_next);
+  else if (vec && out_dtype == kBF16)
+    launch_vec<bf16_t>(grid, stream, resid, a, b, n_terms, w_post, w_next, out, width, eps_post, eps_next);
+  else if (out == nullptr || out_dtype == kF32)
     hipLaunchKernelGGL((add_normed_kernel<float>), grid, block, lds, stream, resid, a, b, n_terms, w_post, w_next,
                        (float*)out, width, eps_post, eps_next);
   else if (out_dtype == kBF16)

@@ -383,7 +383,7 @@ def delta_prepare(proj: torch.Tensor, offsets, heads: int, kv_heads: int, dim: i
     _need(state.dtype is torch.float32 and state.dim() == 2 and state.is_contiguous()
           and state.shape[1] == (taps - 1) * channels + heads * vdim * dim, "state: bad shape")
     _f32(taps_w, "taps", channels * taps)
-    _need(dt_pre.dtype is torch.float32 and dt_pre.is_contiguous() and tuple(dt_pre.shape) == (t, nd), "dt_pre: bad shape")
+    _need(dt_pre.dtype is torch.float32 and dt_pre.stride(1) == 1 and tuple(dt_pre.shape) == (t, nd), "dt_pre: bad shape")
     _f32(dt_bias, "dt_bias", nd)
     _f32(a_log, "A_log", heads)
     dev = proj.device
@@ -394,7 +394,8 @@ def delta_prepare(proj: torch.Tensor, offsets, heads: int, kv_heads: int, dim: i
     decay = torch.empty((t, nd), dtype=torch.float32, device=dev)
     _check(_module("delta_rule").atoma_delta_prepare(
         _p(proj), proj.stride(0), off_q, off_k, off_v, off_b, heads, kv_heads, dim, vdim, taps, _p(token_seq),
-        _p(q_start), _p(state_slots), _p(state), ctypes.c_size_t(state.stride(0)), _p(taps_w), _p(dt_pre), _p(dt_bias),
+        _p(q_start), _p(state_slots), _p(state), ctypes.c_size_t(state.stride(0)), _p(taps_w), _p(dt_pre),
+        dt_pre.stride(0) if t > 1 else nd, _p(dt_bias),
         _p(a_log), _p(qn), _p(kn), _p(vn), _p(beta), _p(decay), t, s, _stream()), "delta_prepare")
     return qn, kn, vn, beta, decay
 
@@ -423,11 +424,13 @@ def delta_out(o: torch.Tensor, gate_pre: torch.Tensor, w: torch.Tensor, eps: flo
     """o / sqrt(mean over a head's columns of o^2 + eps) * w * sigmoid(gate_pre), in ``out_dtype``."""
     _dev(o, gate_pre, w)
     t = o.shape[0]
-    for x, what in ((o, "o"), (gate_pre, "gate")):
-        _need(x.dtype is torch.float32 and x.is_contiguous() and tuple(x.shape) == (t, heads * vdim), f"{what}: bad shape")
+    _need(o.dtype is torch.float32 and o.is_contiguous() and tuple(o.shape) == (t, heads * vdim), "o: bad shape")
+    _need(gate_pre.dtype is torch.float32 and gate_pre.stride(1) == 1 and tuple(gate_pre.shape) == (t, heads * vdim),
+          "gate: bad shape")
     _f32(w, "norm weight", vdim)
     out = torch.empty((t, heads * vdim), dtype=out_dtype, device=o.device)
-    _check(_module("delta_rule").atoma_delta_out(_p(o), _p(gate_pre), _p(w), ctypes.c_float(eps), _p(out),
+    _check(_module("delta_rule").atoma_delta_out(_p(o), _p(gate_pre), gate_pre.stride(0) if t > 1 else heads * vdim,
+                                                 _p(w), ctypes.c_float(eps), _p(out),
                                                  _code(out, "out"), t, heads, vdim, _stream()), "delta_out")
     return out
 
@@ -444,19 +447,19 @@ def route_topk(logits: torch.Tensor, top: int):
     return ids, scores
 
 
-def route_group(ids: torch.Tensor, experts: int):
+def route_group(ids: torch.Tensor, experts: int, tile_m: int = 64):
     """Slots (token, choice) ordered by expert: (perm int32 [slots], offsets int32 [experts + 1], tiles int32
-    [max_tiles, 2] of (expert or -1, first place in perm))."""
+    [max_tiles, 2] of (expert or -1, first place in perm)); a tile holds up to ``tile_m`` (64 or 128) places."""
     _dev(ids)
     _i32(ids, "ids")
     n = ids.numel()
     lib = _module("experts")
-    max_tiles = int(lib.atoma_route_max_tiles(n, experts))
+    max_tiles = int(lib.atoma_route_max_tiles(n, experts, int(tile_m)))
     perm = torch.empty(n, dtype=torch.int32, device=ids.device)
     offsets = torch.empty(experts + 1, dtype=torch.int32, device=ids.device)
     tiles = torch.empty((max_tiles, 2), dtype=torch.int32, device=ids.device)
-    _check(lib.atoma_route_group(_p(ids), n, experts, _p(perm), _p(offsets), _p(tiles), max_tiles, _stream()),
-           "route_group")
+    _check(lib.atoma_route_group(_p(ids), n, experts, _p(perm), _p(offsets), _p(tiles), max_tiles, int(tile_m),
+                                 _stream()), "route_group")
     return perm, offsets, tiles
 
 
@@ -498,10 +501,11 @@ def expert_gemm_mfma_ok(n: int, k: int) -> bool:
 
 
 def expert_gemm_mfma(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, perm, offsets, tiles, top: int, *,
-                     swiglu: bool = False, planes: bool = False) -> None:
+                     swiglu: bool = False, planes: bool = False, tile_m: int = 64) -> None:
     """The grouped product on the matrix cores: a bfloat16 [places, K] in the order of ``perm``, w bfloat16
     [experts, N, K].  ``swiglu``: w's rows in blocks of 16 gate rows and their 16 up rows, out bfloat16
-    [places, N / 2] = silu(gate) * up; else out float32 [places, N] or, with ``planes``, [top, T, N] by slot."""
+    [places, N / 2] = silu(gate) * up; else out float32 [places, N] or, with ``planes``, [top, T, N] by slot.
+    ``tile_m``: what ``route_group`` was told."""
     _dev(a, w, out, perm, offsets, tiles)
     n_slots = perm.numel()
     e, n, k = w.shape
@@ -514,7 +518,7 @@ def expert_gemm_mfma(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, perm, 
     _need(offsets.numel() == e + 1 and tiles.dim() == 2 and tiles.shape[1] == 2, "expert_gemm_mfma: bad grouping")
     _check(_module("experts").atoma_expert_gemm_mfma(
         _p(a), _p(w), _p(out), cols, n, k, _p(perm), _p(offsets), _p(tiles), tiles.shape[0], int(top),
-        n_slots // top if planes else 0, 1 if swiglu else 0, _stream()), "expert_gemm_mfma")
+        n_slots // top if planes else 0, 1 if swiglu else 0, int(tile_m), _stream()), "expert_gemm_mfma")
 
 
 SPLIT_MAX_VOCAB = 262144       # the largest vocabulary whose rows ``sample_packed(split=True)`` cuts into parts

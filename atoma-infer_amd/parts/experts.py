@@ -70,15 +70,19 @@ class RoutedExperts(FeedForward):
     def forward(self, x, ctx):
         t = x.shape[0]
         ids, scores = ops.route_topk(linear(x, self.w_router, torch.float32), self.top)
-        perm, offsets, tiles = ops.route_group(ids.view(-1), self.experts)
         slots = t * self.top
         if self.mfma and x.dtype is torch.bfloat16:
+            # tiles of 128 places where an expert has about a hundred or more (prompts): a weight fragment then
+            # serves twice as many rows
+            tile_m = 128 if slots >= 96 * self.experts else 64
+            perm, offsets, tiles = ops.route_group(ids.view(-1), self.experts, tile_m)
             xs = ops.gather_scale(x, scores.view(-1), perm, self.top)
             h = torch.empty((slots, self.inter), dtype=torch.bfloat16, device=x.device)
-            ops.expert_gemm_mfma(xs, self.w_gate_up, h, perm, offsets, tiles, self.top, swiglu=True)
+            ops.expert_gemm_mfma(xs, self.w_gate_up, h, perm, offsets, tiles, self.top, swiglu=True, tile_m=tile_m)
             out = torch.empty((self.top, t, self.width), dtype=torch.float32, device=x.device)
-            ops.expert_gemm_mfma(h, self.w_down, out, perm, offsets, tiles, self.top, planes=True)
+            ops.expert_gemm_mfma(h, self.w_down, out, perm, offsets, tiles, self.top, planes=True, tile_m=tile_m)
             return out
+        perm, offsets, tiles = ops.route_group(ids.view(-1), self.experts)
         gu = torch.empty((slots, 2 * self.inter), dtype=x.dtype, device=x.device)
         ops.expert_gemm(x, self.w_gate_up, gu, perm, offsets, tiles, self.top, gather=True, scale=scores.view(-1))
         h = ops.swiglu(gu)

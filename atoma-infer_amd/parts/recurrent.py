@@ -54,7 +54,7 @@ class GatedDeltaRule(Mixer):
         self.off_b = self.off_v + self.nv
         self.off_a1 = self.off_b + self.heads
         self.off_g1 = None
-        self.w_in = self.w_a2 = self.w_g2 = self.w_o = self.w_o_tiled = None
+        self.w_in = self.w_ag = self.w_o = self.w_o_tiled = None
         self.taps_w = self.a_log = self.dt_bias = self.norm_w = None
 
     def graph_safe(self) -> bool:
@@ -87,10 +87,16 @@ class GatedDeltaRule(Mixer):
         if pad:
             parts.append(torch.zeros((pad, self.width), dtype=dt, device=device))
         self.w_in = torch.cat(parts, dim=0).contiguous()
-        self.w_a2, self.w_g2 = get("a2").to(device).contiguous(), get("g2").to(device).contiguous()
-        if self.w_a2.shape[1] != self.decay_rank or self.w_g2.shape[1] != self.gate_rank:
+        a2, g2 = get("a2"), get("g2")
+        if a2.shape[1] != self.decay_rank or g2.shape[1] != self.gate_rank:
             raise ValueError(f"the halves of a low-rank map do not fit: a1 {tuple(ws[4].shape)} and a2 "
-                             f"{tuple(self.w_a2.shape)}, g1 {tuple(ws[5].shape)} and g2 {tuple(self.w_g2.shape)}")
+                             f"{tuple(a2.shape)}, g1 {tuple(ws[5].shape)} and g2 {tuple(g2.shape)}")
+        # the second halves of both low-rank maps as one matrix, [[a2, 0], [0, g2]], for one product over the
+        # neighbouring columns of a1's and g1's results (the zeros add nothing)
+        dt2 = a2.dtype if a2.dtype is g2.dtype else torch.float32
+        self.w_ag = torch.zeros((self.nd + self.nv, self.decay_rank + self.gate_rank), dtype=dt2, device=device)
+        self.w_ag[: self.nd, : self.decay_rank] = a2.to(device=device, dtype=dt2)
+        self.w_ag[self.nd:, self.decay_rank:] = g2.to(device=device, dtype=dt2)
         self.w_o = get("o").to(device).contiguous()
         f32 = dict(device=device, dtype=torch.float32)
         self.taps_w = torch.cat([get(n + ".conv").to(**f32) for n in ("q", "k", "v")], dim=0).contiguous()
@@ -102,14 +108,14 @@ class GatedDeltaRule(Mixer):
             self.w_o_tiled = gemm_bf16.tile_copies_resid(self.w_o)
 
     def device_bytes(self) -> int:
-        return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_a2, self.w_g2, self.w_o))
+        return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_ag, self.w_o))
 
     def forward(self, x, ctx, cache):
         state = cache.state
         proj = linear(x, self.w_in, torch.float32)
-        # the second halves of the two low-rank maps read their slices of the float32 projection as they are
-        dt_pre = linear(proj[:, self.off_a1: self.off_a1 + self.decay_rank], self.w_a2, torch.float32)
-        gate_pre = linear(proj[:, self.off_g1: self.off_g1 + self.gate_rank], self.w_g2, torch.float32)
+        # the second halves of the two low-rank maps read their columns of the float32 projection as they are
+        pre = linear(proj[:, self.off_a1: self.off_g1 + self.gate_rank], self.w_ag, torch.float32)
+        dt_pre, gate_pre = pre[:, : self.nd], pre[:, self.nd:]
         qn, kn, vn, beta, decay = ops.delta_prepare(
             proj, (self.off_q, self.off_k, self.off_v, self.off_b), self.heads, self.kv_heads, self.dim, self.vdim,
             self.taps, ctx.token_seq, ctx.q_start, ctx.state_slots, state, self.taps_w, dt_pre, self.dt_bias, self.a_log)

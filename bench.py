@@ -12,6 +12,11 @@ token ids, a batch of 8, and a maximum context of 8192.  It prints ONE JSON line
 and decode throughput at batch 1 and 64; the read and copy bandwidth and the MFMA rate that this GPU delivers,
 measured by small probes, stand beside the published peaks (which stay the yardstick of every fraction).
 
+``--compare somesun`` measures the Somesun decoder (attention with chunks and sinks beside a gated delta rule, routed
+experts) at layer sizes that resemble a real model's, beside the Llama of equal width, heads and active feed-forward
+width: prefill of 2,048 tokens and decode steps at batch 1, 8 and 64 through the same engine, ONE line of its own
+(``--sizes 1b|3b`` picks the pair, ``--layers`` how many layers of each, 4 by default; ``--only`` one of the two).
+
 ``--workload`` runs one of the other two workloads instead and prints ONE line of its own:
 ``serve3b``: Llama-3.2-3B sizes, 64 requests with prompt lengths uniform in [128, 4096] (seeded), 256 generated tokens
 each, continuous batching with chunked prefill under 2,048 tokens a step; ``long8b``: Llama-3.1-8B sizes, 16 requests
@@ -170,6 +175,89 @@ def serve_run(model, n_req, lo, hi, out_tokens, budget, seed=3):
             "step_p99_ms": times[int(len(times) * 0.99)] * 1e3}
 
 
+def somesun_like(llama: dict, layers: int) -> dict:
+    """The Somesun configuration beside ``llama``: the same width, vocabulary, attention heads and head size; chunks of
+    1,024 positions; a recurrent branch of half as many heads of 128 x 128; experts of a quarter (1b) or half (3b) of
+    the dense feed-forward's width of which as many are chosen as make up that width."""
+    w, nh, nkv = llama["hidden_size"], llama["num_attention_heads"], llama["num_key_value_heads"]
+    hd = w // nh
+    rh = w // 256
+    ff = 2048 if w <= 2048 else 4096
+    top = llama["intermediate_size"] // ff
+    layer = {"type": "parallel",
+             "mixer": {"left": {"dim": hd, "heads": nh, "kv_heads": nkv, "vdim": hd, "scale": hd ** -0.5,
+                                "mask": {"size": 1024}, "rot": {"base": 500000.0, "dims": hd}},
+                       "right": {"dim": 128, "heads": rh, "kv_heads": rh // 2, "vdim": 128, "conv": 4,
+                                 "decay_rank": 64, "gate_rank": 64},
+                       "left_scale": 0.5, "right_scale": 0.5},
+             "mlp": {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": 8 * top, "top": top}}}
+    return {"architecture": "Somesun", "layers": [layer] * layers, "norm": {"eps": 1e-5},
+            "vocab": llama["vocab_size"], "width": w, "max_positions": llama["max_position_embeddings"]}
+
+
+def step_bytes_somesun(cfg: dict, batch: int, ctx: float) -> float:
+    """Bytes a decode step of ``batch`` requests at context ``ctx`` has to read (and, for the state, write): every
+    dense matrix once, the experts that ``batch`` tokens are expected to choose between them, the keys and values of
+    each request's current chunk, the recurrent state twice."""
+    total = 2.0 * cfg["vocab"] * cfg["width"]
+    w = cfg["width"]
+    for l in cfg["layers"]:
+        a, r, m = l["mixer"]["left"], l["mixer"]["right"], l["mlp"]
+        total += 2.0 * w * (2 * a["heads"] + a["kv_heads"]) * a["dim"]
+        rq, rv = r["kv_heads"] * r["dim"], r["heads"] * r["vdim"]
+        total += 2.0 * (w * (2 * rq + 2 * rv + r["heads"] + r["decay_rank"] + r["gate_rank"])
+                        + r["decay_rank"] * r["heads"] * r["dim"] + r["gate_rank"] * rv)
+        e, top = m["router"]["experts"], m["router"]["top"]
+        chosen = e * (1.0 - (1.0 - top / e) ** batch)
+        total += 2.0 * w * e + chosen * 2.0 * 3 * w * m["expert"]["ff"]
+        seen = min(ctx, a["mask"]["size"] / 2.0)
+        total += batch * (2.0 * 2 * a["kv_heads"] * a["dim"] * seen + 2 * 4.0 * r["heads"] * r["dim"] * r["vdim"])
+    return total
+
+
+def compare_main(args) -> int:
+    import torch
+    import atoma_infer_amd  # noqa: F401
+    from atoma_infer_amd.cache import plan_cache
+    from atoma_infer_amd.models import random_model
+    sizes = args.sizes if args.sizes in ("1b", "3b") else "1b"
+    layers = args.layers or 4
+    llama = dict(LLAMA_1B, **OTHER_SIZES.get(sizes, {}), num_hidden_layers=layers)
+    sun = somesun_like(llama, layers)
+    out = {}
+    for name, cfg in (("llama", llama), ("somesun", sun)):
+        if args.only and args.only != name:
+            continue
+        log(f"{name}: building {layers} layers at {sizes} sizes (random weights) ...")
+        model = random_model(cfg, seed=0, dtype="bfloat16", stored="bfloat16")
+        pre_s = prefill_run(model, args.prefill_tokens, 4, args.context)
+        res = {"prefill_ms": round(pre_s * 1e3, 3), "prefill_tok_s": round(args.prefill_tokens / pre_s, 1)}
+        kv = plan_cache(model.spec).bytes_per_token(2)
+        for b in (1, 8, 64):
+            st = min(args.steps, 64)
+            log(f"{name}: decode at batch {b} ...")
+            d, ctx = decode_run(model, b, args.prompt_len, st, min(args.warmup, 4), args.context)
+            nbytes = step_bytes_somesun(sun, b, ctx) if name == "somesun" else model.weight_bytes() + kv * ctx * b
+            res[f"decode_b{b}_tok_s"] = round(b * st / d, 1)
+            res[f"decode_b{b}_ms"] = round(d / st * 1e3, 4)
+            res[f"decode_b{b}_frac"] = round(nbytes / (d / st) / 1e9 / HBM_PEAK_GBS, 4)
+        out[name] = res
+        del model
+        torch.cuda.empty_cache()
+    l = sun["layers"][0]
+    line = {"metric": f"Somesun beside Llama at {sizes} layer sizes, {layers} layers each: prefill of "
+                      f"{args.prefill_tokens} tokens, decode at batch 1, 8, 64 ({args.prompt_len}-token prompts)",
+            "unit": "tokens/s, ms a step, fraction of 8 TB/s", "n_gpus": 1, "dtype": "bf16",
+            "data": "synthetic (uniform random token ids, random weights)",
+            "config": {"width": sun["width"], "vocab": sun["vocab"], "layers": layers, "left": l["mixer"]["left"],
+                       "right": l["mixer"]["right"], "mlp": l["mlp"],
+                       "llama": {k: llama[k] for k in ("hidden_size", "intermediate_size", "num_attention_heads",
+                                                        "num_key_value_heads")}},
+            **out}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def workload_main(args) -> int:
     import atoma_infer_amd  # noqa: F401
     from atoma_infer_amd.models import random_model
@@ -224,6 +312,9 @@ def main() -> int:
     ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--workload", choices=["decode", *WORKLOADS], default="decode",
                     help="decode: the default run; serve3b, long8b: the other two workloads, one line of their own")
+    ap.add_argument("--compare", choices=["somesun"], default=None,
+                    help="measure that design at --sizes (1b, 3b) beside the Llama of equal sizes, one line of its own")
+    ap.add_argument("--only", choices=["llama", "somesun"], default=None, help="with --compare: one of the two models")
     ap.add_argument("--requests", type=int, default=0, help="requests of a --workload run (default: the workload's)")
     ap.add_argument("--no-peaks", action="store_true", help="skip the probes of what the GPU delivers")
     ap.add_argument("--chain-floors", action="store_true",
@@ -241,6 +332,8 @@ def main() -> int:
         from atoma_infer_amd.kernels.ops import measure_chain_floors
         print(json.dumps({"chain_floors": measure_chain_floors(), "unit": "us a kernel"}), flush=True)
         return 0
+    if args.compare:
+        return compare_main(args)
     if args.workload != "decode":
         return workload_main(args)
     if args.prompt_len + args.steps + args.warmup + 2 * args.batch * (-(-args.prompt_len // 2048)) + 8 > args.context:

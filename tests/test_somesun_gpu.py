@@ -156,7 +156,7 @@ def test_routed_experts_alone(experts, top, ff, dtype):
     # path, run float32 multiply-adds)
     assert part.mfma == (dtype is torch.bfloat16 and ff % 32 == 0)
     g = torch.Generator().manual_seed(experts)
-    for t in (1, 3, 150):          # one row tile, and experts whose rows fill more than one
+    for t in (1, 3, 150, 700):     # one row tile, experts whose rows fill more than one, tiles of 128 places
         h = torch.randn(t, width, generator=g).to(torch.bfloat16).float()
         want = ps.routed_experts(h.double(), {"m." + k: v.double() for k, v in w.items()}, "m.",
                                  {"router": {"experts": experts, "top": top}})
