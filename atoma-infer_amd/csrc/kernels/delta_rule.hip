@@ -37,7 +37,8 @@ delta_prepare_kernel(const float* __restrict__ proj, DeltaShape sh, const int32_
                      const float* __restrict__ state, size_t state_stride, const float* __restrict__ taps_w,
                      const float* __restrict__ dt_pre, int ld_dt, const float* __restrict__ dt_bias,
                      const float* __restrict__ a_log, float* __restrict__ qn, float* __restrict__ kn,
-                     float* __restrict__ vn, float* __restrict__ beta, float* __restrict__ decay) {
+                     float* __restrict__ vn, float* __restrict__ beta, float* __restrict__ decay,
+                     float* __restrict__ kq) {
   extern __shared__ float act[];       // the token's channels after convolution and SiLU
   const int t = blockIdx.x;
   const int e = token_seq[t];
@@ -71,14 +72,22 @@ delta_prepare_kernel(const float* __restrict__ proj, DeltaShape sh, const int32_
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const float q_scale = 1.0f / sqrtf((float)sh.dim);
   for (int hh = wave; hh < 2 * sh.kv_heads; hh += 4) {
-    const float* x = act + (size_t)hh * sh.dim;
+    float* x = act + (size_t)hh * sh.dim;
     float ss = 0.f;
     for (int i = lane; i < sh.dim; i += 64) ss += x[i] * x[i];
     ss = wave_sum(ss);
     const bool is_q = hh < sh.kv_heads;
     const float inv = (is_q ? q_scale : 1.0f) / sqrtf(ss + 1e-6f);
     float* dst = (is_q ? qn : kn) + (size_t)t * nqk + (size_t)(is_q ? hh : hh - sh.kv_heads) * sh.dim;
-    for (int i = lane; i < sh.dim; i += 64) dst[i] = x[i] * inv;
+    for (int i = lane; i < sh.dim; i += 64) dst[i] = act[(size_t)hh * sh.dim + i] = x[i] * inv;
+  }
+  __syncthreads();
+  // k . q of every q/k head, which the recurrence's read-out needs once a token
+  for (int hh = wave; hh < sh.kv_heads; hh += 4) {
+    float d = 0.f;
+    for (int i = lane; i < sh.dim; i += 64) d = fmaf(act[(size_t)hh * sh.dim + i], act[(size_t)(sh.kv_heads + hh) * sh.dim + i], d);
+    d = wave_sum(d);
+    if (lane == 0) kq[(size_t)t * sh.kv_heads + hh] = d;
   }
   for (int c = threadIdx.x; c < nv; c += 256) vn[(size_t)t * nv + c] = act[2 * nqk + c];
 }
@@ -111,20 +120,20 @@ __device__ __forceinline__ float row16_sum(float x) {
 }
 
 // R: rows of S a lane holds.  16 lanes (a DPP row) share a column of S, so dim <= 16 R; a wave holds 4 columns, a
-// workgroup of four waves 16.  The tokens' q, k, decay (for the head), v (for the 16 columns) and beta pass LDS in
-// blocks of TB tokens: the next block is fetched from memory while this one is worked on, so the walk over the tokens
-// waits for LDS only.
+// workgroup of four waves 16.  The tokens' q, k, decay (for the head), v (for the 16 columns), beta and k . q pass
+// LDS in blocks of TB tokens: the next block is fetched from memory while this one is worked on, so the walk over the
+// tokens waits for LDS only.
 template <int R>
 __global__ void __launch_bounds__(256)
 delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vn,
-                  const float* __restrict__ beta, const float* __restrict__ decay, DeltaShape sh,
-                  const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
+                  const float* __restrict__ beta, const float* __restrict__ decay, const float* __restrict__ kq,
+                  DeltaShape sh, const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
                   float* __restrict__ state, size_t state_stride, size_t s_offset, float* __restrict__ o) {
   constexpr int DP = 16 * R;                   // dim rounded up; rows beyond dim hold zeros
   constexpr int TB = R <= 8 ? 16 : 8;          // tokens a block
   constexpr int PER = TB * DP / 256;           // elements of q (k, decay) a thread fetches a block
   __shared__ float sq[2][TB][DP], sk[2][TB][DP], sg[2][TB][DP];
-  __shared__ float sv[2][TB][16], sb[2][TB];
+  __shared__ float sv[2][TB][16], sb[2][TB], skq[2][TB];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int part = lane & 15;
   const int col_local = wave * 4 + (lane >> 4);
@@ -142,8 +151,8 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, co
   for (int r = 0; r < R; ++r) s[r] = (col_ok && i0 + r < dim) ? sp[r] : 0.f;
 
   const int nqk = sh.kv_heads * dim, nd = sh.heads * dim, nv = sh.heads * vdim;
-  float pq[PER], pk[PER], pg[PER], pv = 0.f, pb = 0.f;
-  // block b's share of this thread: element idx = tid + j * 256 of [TB][DP]; v: thread tid of [TB][16]; beta: tid < TB
+  float pq[PER], pk[PER], pg[PER], pv = 0.f, pb = 0.f, pkq = 0.f;
+  // block b's share of this thread: element idx = tid + j * 256 of [TB][DP]; v: thread tid of [TB][16]; beta, k . q: tid < TB
   auto fetch = [&](int b) {
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
@@ -160,7 +169,11 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, co
       const int n = b * TB + tok;
       pv = (n < count && c < vdim) ? vn[(size_t)(first + n) * nv + (size_t)h * vdim + c] : 0.f;
     }
-    if (tid < TB) pb = (b * TB + tid < count) ? beta[(size_t)(first + b * TB + tid) * sh.heads + h] : 0.f;
+    if (tid < TB) {
+      const bool ok = b * TB + tid < count;
+      pb = ok ? beta[(size_t)(first + b * TB + tid) * sh.heads + h] : 0.f;
+      pkq = ok ? kq[(size_t)(first + b * TB + tid) * sh.kv_heads + kv] : 0.f;
+    }
   };
   auto stash = [&](int buf) {
 #pragma unroll
@@ -171,7 +184,7 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, co
       sg[buf][tok][i] = pg[j];
     }
     if (tid < TB * 16) sv[buf][tid >> 4][tid & 15] = pv;
-    if (tid < TB) sb[buf][tid] = pb;
+    if (tid < TB) sb[buf][tid] = pb, skq[buf][tid] = pkq;
   };
   const int blocks = (count + TB - 1) / TB;
   if (blocks > 0) {
@@ -183,24 +196,23 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, co
     const int buf = b & 1;
     if (b + 1 < blocks) fetch(b + 1);
     const int n_tok = min(TB, count - b * TB);
+#pragma unroll 2
     for (int tok = 0; tok < n_tok; ++tok) {
-      float d1 = 0.f, d2 = 0.f, kq = 0.f;
+      float d1 = 0.f, d2 = 0.f;
       float kr[R];
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const float g = sg[buf][tok][i0 + r], q = sq[buf][tok][i0 + r];
         kr[r] = sk[buf][tok][i0 + r];
-        s[r] *= g;
+        s[r] *= sg[buf][tok][i0 + r];
         d1 = fmaf(s[r], kr[r], d1);
-        d2 = fmaf(s[r], q, d2);
-        kq = fmaf(kr[r], q, kq);
+        d2 = fmaf(s[r], sq[buf][tok][i0 + r], d2);
       }
       d1 = row16_sum(d1);
       d2 = row16_sum(d2);
-      kq = row16_sum(kq);
       const float u = sb[buf][tok] * (sv[buf][tok][col_local] - d1);
       // o = S_new^T q with S_new = diag(g) S + k u^T
-      if (part == 0 && col_ok) o[(size_t)(first + b * TB + tok) * nv + (size_t)h * vdim + col] = fmaf(u, kq, d2);
+      if (part == 0 && col_ok)
+        o[(size_t)(first + b * TB + tok) * nv + (size_t)h * vdim + col] = fmaf(u, skq[buf][tok], d2);
 #pragma unroll
       for (int r = 0; r < R; ++r) s[r] = fmaf(kr[r], u, s[r]);
     }
@@ -242,7 +254,7 @@ extern "C" int atoma_delta_prepare(const float* proj, int ldp, int off_q, int of
                                    size_t state_stride, const float* taps_w, const float* dt_pre, int ld_dt,
                                    const float* dt_bias,
                                    const float* a_log, float* qn, float* kn, float* vn, float* beta, float* decay,
-                                   int n_tokens, int n_entries, hipStream_t stream) {
+                                   float* kq, int n_tokens, int n_entries, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   DeltaShape sh{heads, kv_heads, dim, vdim, taps, ldp, off_q, off_k, off_v, off_b};
   if (!shape_ok(sh) || n_entries <= 0 || n_entries > 65535) return ATOMA_ERR_SHAPE;
@@ -251,7 +263,7 @@ extern "C" int atoma_delta_prepare(const float* proj, int ldp, int off_q, int of
   if ((size_t)channels * sizeof(float) > 60 * 1024) return ATOMA_ERR_SHAPE;
   hipLaunchKernelGGL(delta_prepare_kernel, dim3(n_tokens, 2), dim3(256), channels * sizeof(float), stream, proj, sh,
                      token_seq, q_start, state_slots, state, state_stride, taps_w, dt_pre, ld_dt, dt_bias, a_log, qn, kn, vn,
-                     beta, decay);
+                     beta, decay, kq);
   ATOMA_LAUNCH_CHECK();
   if (taps > 1) {
     hipLaunchKernelGGL(delta_conv_state_kernel, dim3((channels + 255) / 256, n_entries), dim3(256), 0, stream, proj, sh,
@@ -262,7 +274,7 @@ extern "C" int atoma_delta_prepare(const float* proj, int ldp, int off_q, int of
 }
 
 extern "C" int atoma_delta_scan(const float* qn, const float* kn, const float* vn, const float* beta,
-                                const float* decay, int heads, int kv_heads, int dim, int vdim, int taps,
+                                const float* decay, const float* kq, int heads, int kv_heads, int dim, int vdim, int taps,
                                 const int32_t* q_start, const int32_t* state_slots, float* state, size_t state_stride,
                                 int n_entries, float* o, hipStream_t stream) {
   if (n_entries <= 0) return 0;
@@ -271,7 +283,7 @@ extern "C" int atoma_delta_scan(const float* qn, const float* kn, const float* v
   const size_t s_offset = (size_t)(taps - 1) * (2 * kv_heads * dim + heads * vdim);
   dim3 grid((vdim + 15) / 16, heads, n_entries), block(256);
 #define ATOMA_SCAN(R_)                                                                                            \
-  hipLaunchKernelGGL((delta_scan_kernel<R_>), grid, block, 0, stream, qn, kn, vn, beta, decay, sh, q_start,       \
+  hipLaunchKernelGGL((delta_scan_kernel<R_>), grid, block, 0, stream, qn, kn, vn, beta, decay, kq, sh, q_start,   \
                      state_slots, state, state_stride, s_offset, o)
   if (dim <= 16) ATOMA_SCAN(1);
   else if (dim <= 32) ATOMA_SCAN(2);

@@ -170,7 +170,9 @@ gather_scale_kernel(const uint16_t* __restrict__ x, int ldx, const float* __rest
 
 constexpr int kLdsRow = 64 + 8;     // bfloat16 elements a row of the activations' tile takes in LDS (padded)
 
-template <bool SWIGLU, int TM>
+// NS: blocks of 16 rows of the weight a wave takes (2 or 4: a fragment of the activations read from LDS then feeds as
+// many products, and LDS is what bounds a tile of 128 places)
+template <bool SWIGLU, int TM, int NS>
 __global__ void __launch_bounds__(256)
 expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, void* __restrict__ c, int ldc,
                         int N, int K, const int32_t* __restrict__ perm, const int32_t* __restrict__ offsets,
@@ -185,31 +187,31 @@ expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restri
   const int msub = (rows + 15) >> 4;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
-  const int n_base = blockIdx.x * 128 + wave * 32;
+  const int n_base = blockIdx.x * (64 * NS) + wave * (16 * NS);
   // (a wave whose columns lie beyond N still joins the barriers below; its rows are clamped and never stored)
   const uint16_t* we = w + (size_t)e * N * K;
-  const uint16_t* wp[2];
+  const uint16_t* wp[NS];
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
+  for (int s = 0; s < NS; ++s) {
     int n = n_base + s * 16 + r16;
     if (n > N - 1) n = N - 1;
     wp[s] = we + (size_t)n * K + kg * 8;
   }
-  f32x4 acc[2][MS];
+  f32x4 acc[NS][MS];
 #pragma unroll
-  for (int s = 0; s < 2; ++s)
+  for (int s = 0; s < NS; ++s)
 #pragma unroll
     for (int m = 0; m < MS; ++m) acc[s][m] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // The operands of a step are asked for a step ahead: the weight's fragments wait in registers, the activations' pieces
   // too, until the tile of the step before has been read and they may go to LDS.
-  bf16x8 wf[2][2], wn[2][2];
+  bf16x8 wf[2][NS], wn[2][NS];
   uint4 ar[AP];
-  auto fetch = [&](int k0, bf16x8 (&dst)[2][2]) {
+  auto fetch = [&](int k0, bf16x8 (&dst)[2][NS]) {
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
+      for (int s = 0; s < NS; ++s) {
         // (K is a multiple of 32: the last step may have its first half only)
         if (k0 + kk * 32 < K) dst[kk][s] = *reinterpret_cast<const bf16x8*>(wp[s] + k0 + kk * 32);
         else dst[kk][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
@@ -238,7 +240,7 @@ expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restri
         if (m < msub) {
           const bf16x8 af = *reinterpret_cast<const bf16x8*>(at + (m * 16 + r16) * kLdsRow + kk * 32 + kg * 8);
 #pragma unroll
-          for (int s = 0; s < 2; ++s)
+          for (int s = 0; s < NS; ++s)
             acc[s][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[kk][s], af, acc[s][m], 0, 0, 0);
         }
       }
@@ -246,29 +248,32 @@ expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restri
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-      for (int s = 0; s < 2; ++s) wf[kk][s] = wn[kk][s];
+      for (int s = 0; s < NS; ++s) wf[kk][s] = wn[kk][s];
   }
-  // lane: place m * 16 + r16 of the tile, columns kg * 4 .. + 3 of each of its two blocks of 16 rows of the weight
+  // lane: place m * 16 + r16 of the tile, columns kg * 4 .. + 3 of each of its NS blocks of 16 rows of the weight
 #pragma unroll
   for (int m = 0; m < MS; ++m) {
     const int r = m * 16 + r16;
     if (m >= msub || r >= rows) continue;
     const int place = row0 + r;
     if constexpr (SWIGLU) {
-      const int n0 = n_base / 2 + kg * 4;      // outputs: one for every pair of a gate row and an up row
-      uint16_t* dst = (uint16_t*)c + (size_t)place * ldc + n0;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (n_base + 16 + kg * 4 + i < N) {
-          const float g = acc[0][m][i];
-          dst[i] = f32_to_bf16_bits(g / (1.0f + expf(-g)) * acc[1][m][i]);
+      for (int s = 0; s < NS; s += 2) {        // blocks come in pairs: 16 gate rows, then their 16 up rows
+        const int n0 = (n_base + s * 16) / 2 + kg * 4;      // outputs: one for every pair of a gate row and an up row
+        uint16_t* dst = (uint16_t*)c + (size_t)place * ldc + n0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (n_base + s * 16 + 16 + kg * 4 + i < N) {
+            const float g = acc[s][m][i];
+            dst[i] = f32_to_bf16_bits(g / (1.0f + expf(-g)) * acc[s + 1][m][i]);
+          }
         }
       }
     } else {
       const int slot = perm[place];
       const size_t row = plane_rows > 0 ? (size_t)(slot % top) * plane_rows + slot / top : (size_t)place;
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
+      for (int s = 0; s < NS; ++s) {
         const int n0 = n_base + s * 16 + kg * 4;
         float* dst = (float*)c + row * ldc + n0;
 #pragma unroll
@@ -298,14 +303,15 @@ extern "C" int atoma_expert_gemm_mfma(const void* a, const void* w, void* c, int
   if (K <= 0 || K % 32 || N % 32 || (tile_m != 64 && tile_m != 128) || top <= 0 || max_tiles > 65535 || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) ||
       ldc < (swiglu ? N / 2 : N))
     return ATOMA_ERR_SHAPE;
-  dim3 grid((N + 127) / 128, max_tiles), block(256);
-#define ATOMA_EGM(SW, TM_)                                                                                       \
-  hipLaunchKernelGGL((expert_gemm_mfma_kernel<SW, TM_>), grid, block, 0, stream, (const uint16_t*)a,             \
+  const int ns = 2;      // (four blocks a wave measured slower for tiles of 128 places: 467 against 336 us)
+  dim3 grid((N + 64 * ns - 1) / (64 * ns), max_tiles), block(256);
+#define ATOMA_EGM(SW, TM_, NS_)                                                                                  \
+  hipLaunchKernelGGL((expert_gemm_mfma_kernel<SW, TM_, NS_>), grid, block, 0, stream, (const uint16_t*)a,        \
                      (const uint16_t*)w, c, ldc, N, K, perm, offsets, tiles, top, plane_rows)
-  if (swiglu && tile_m == 64) ATOMA_EGM(true, 64);
-  else if (swiglu) ATOMA_EGM(true, 128);
-  else if (tile_m == 64) ATOMA_EGM(false, 64);
-  else ATOMA_EGM(false, 128);
+  if (swiglu && tile_m == 64) ATOMA_EGM(true, 64, 2);
+  else if (swiglu) ATOMA_EGM(true, 128, 2);
+  else if (tile_m == 64) ATOMA_EGM(false, 64, 2);
+  else ATOMA_EGM(false, 128, 2);
 #undef ATOMA_EGM
   ATOMA_LAUNCH_CHECK();
   return 0;

@@ -365,7 +365,7 @@ def qk_norm_rope(qk: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tens
 def delta_prepare(proj: torch.Tensor, offsets, heads: int, kv_heads: int, dim: int, vdim: int, taps: int,
                   token_seq: torch.Tensor, q_start: torch.Tensor, state_slots: torch.Tensor, state: torch.Tensor,
                   taps_w: torch.Tensor, dt_pre: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor):
-    """The inputs of the gated delta rule for every token (see delta_rule.hip): (q, k, v, beta, decay), all float32,
+    """The inputs of the gated delta rule for every token (see delta_rule.hip): (q, k, v, beta, decay, k . q), all float32,
     from ``proj`` float32 [T, ld] whose columns ``offsets`` = (q, k, v, b) name; the convolution's state rows of each
     entry's request are read and then replaced."""
     _dev(proj, token_seq, q_start, state_slots, state, taps_w, dt_pre, dt_bias, a_log)
@@ -392,21 +392,23 @@ def delta_prepare(proj: torch.Tensor, offsets, heads: int, kv_heads: int, dim: i
     vn = torch.empty((t, nv), dtype=torch.float32, device=dev)
     beta = torch.empty((t, heads), dtype=torch.float32, device=dev)
     decay = torch.empty((t, nd), dtype=torch.float32, device=dev)
+    kq = torch.empty((t, kv_heads), dtype=torch.float32, device=dev)
     _check(_module("delta_rule").atoma_delta_prepare(
         _p(proj), proj.stride(0), off_q, off_k, off_v, off_b, heads, kv_heads, dim, vdim, taps, _p(token_seq),
         _p(q_start), _p(state_slots), _p(state), ctypes.c_size_t(state.stride(0)), _p(taps_w), _p(dt_pre),
         dt_pre.stride(0) if t > 1 else nd, _p(dt_bias),
-        _p(a_log), _p(qn), _p(kn), _p(vn), _p(beta), _p(decay), t, s, _stream()), "delta_prepare")
-    return qn, kn, vn, beta, decay
+        _p(a_log), _p(qn), _p(kn), _p(vn), _p(beta), _p(decay), _p(kq), t, s, _stream()), "delta_prepare")
+    return qn, kn, vn, beta, decay, kq
 
 
-def delta_scan(qn, kn, vn, beta, decay, heads: int, kv_heads: int, dim: int, vdim: int, taps: int,
+def delta_scan(qn, kn, vn, beta, decay, kq, heads: int, kv_heads: int, dim: int, vdim: int, taps: int,
                q_start: torch.Tensor, state_slots: torch.Tensor, state: torch.Tensor) -> torch.Tensor:
     """The recurrence over every entry's tokens, from and into the requests' state rows; returns o float32 [T, heads vdim]."""
-    _dev(qn, kn, vn, beta, decay, q_start, state_slots, state)
+    _dev(qn, kn, vn, beta, decay, kq, q_start, state_slots, state)
     t, s = qn.shape[0], state_slots.numel()
     nqk, nv, nd = kv_heads * dim, heads * vdim, heads * dim
-    for x, n, what in ((qn, nqk, "q"), (kn, nqk, "k"), (vn, nv, "v"), (beta, heads, "beta"), (decay, nd, "decay")):
+    for x, n, what in ((qn, nqk, "q"), (kn, nqk, "k"), (vn, nv, "v"), (beta, heads, "beta"), (decay, nd, "decay"),
+                       (kq, kv_heads, "k . q")):
         _need(x.dtype is torch.float32 and x.is_contiguous() and tuple(x.shape) == (t, n), f"{what}: bad shape")
     _i32(q_start, "q_start", s + 1)
     _i32(state_slots, "state_slots", s)
@@ -414,7 +416,7 @@ def delta_scan(qn, kn, vn, beta, decay, heads: int, kv_heads: int, dim: int, vdi
           and state.shape[1] == (taps - 1) * (2 * nqk + nv) + heads * vdim * dim, "state: bad shape")
     o = torch.empty((t, nv), dtype=torch.float32, device=qn.device)
     _check(_module("delta_rule").atoma_delta_scan(
-        _p(qn), _p(kn), _p(vn), _p(beta), _p(decay), heads, kv_heads, dim, vdim, taps, _p(q_start), _p(state_slots),
+        _p(qn), _p(kn), _p(vn), _p(beta), _p(decay), _p(kq), heads, kv_heads, dim, vdim, taps, _p(q_start), _p(state_slots),
         _p(state), ctypes.c_size_t(state.stride(0)), s, _p(o), _stream()), "delta_scan")
     return o
 

@@ -116,10 +116,10 @@ class GatedDeltaRule(Mixer):
         # the second halves of the two low-rank maps read their columns of the float32 projection as they are
         pre = linear(proj[:, self.off_a1: self.off_g1 + self.gate_rank], self.w_ag, torch.float32)
         dt_pre, gate_pre = pre[:, : self.nd], pre[:, self.nd:]
-        qn, kn, vn, beta, decay = ops.delta_prepare(
+        qn, kn, vn, beta, decay, kq = ops.delta_prepare(
             proj, (self.off_q, self.off_k, self.off_v, self.off_b), self.heads, self.kv_heads, self.dim, self.vdim,
             self.taps, ctx.token_seq, ctx.q_start, ctx.state_slots, state, self.taps_w, dt_pre, self.dt_bias, self.a_log)
-        o = ops.delta_scan(qn, kn, vn, beta, decay, self.heads, self.kv_heads, self.dim, self.vdim, self.taps,
+        o = ops.delta_scan(qn, kn, vn, beta, decay, kq, self.heads, self.kv_heads, self.dim, self.vdim, self.taps,
                            ctx.q_start, ctx.state_slots, state)
         y = ops.delta_out(o, gate_pre, self.norm_w, self.norm_eps, self.heads, self.vdim, x.dtype)
         return linear_delta(y, self.w_o, None, self.w_o_tiled)
