@@ -28,6 +28,8 @@ class GroupGeometry:
     page_size: int
     num_pages: int
     window: Optional[int] = None
+    #: chunks of this many positions instead of a window: a token sees the keys of its own chunk only
+    chunk: Optional[int] = None
 
 
 _lib = None
@@ -81,7 +83,9 @@ class CacheManager:
         self.num_state_slots = int(num_state_slots)
         lib = _host()
         ps, npg = _i32(g.page_size for g in groups), _i32(g.num_pages for g in groups)
-        win = _i32((g.window or 0) for g in groups)
+        if any(g.window and g.chunk for g in groups):
+            raise CacheError("a group keeps a window or chunks, not both")
+        win = _i32((-g.chunk if g.chunk else (g.window or 0)) for g in groups)      # chunks travel as negative windows
         self._h = lib.cm_create(len(self.groups), ps.ctypes.data, npg.ctypes.data, win.ctypes.data,
                                 self.num_state_slots)
         if not self._h:

@@ -101,7 +101,7 @@ class CachePool:
                                       device=device))
             self.v.append(torch.zeros((len(g.calls), n, cs.kv_heads, page_size * cs.value_elements), dtype=dtype,
                                       device=device) if cs.value_elements else None)
-            geometry.append(GroupGeometry(page_size, n, cs.window))
+            geometry.append(GroupGeometry(page_size, n, cs.window, cs.chunk))
         self.states = {pos: torch.zeros((num_state_slots, *shape), dtype=getattr(torch, dt), device=device)
                        for pos, (shape, dt) in plan.states.items()}
         self.manager = CacheManager(geometry, num_state_slots)

@@ -20,6 +20,10 @@ struct Group {
   int page_size = 0;
   int num_pages = 0;
   int window = 0;  // 0: keep everything
+  // false: a token sees the last `window` keys.  true: it sees the keys of its own chunk of `window` positions
+  // (chunks count from the request's first position), so everything before the chunk of the next token is dead.
+  // Either way a request never needs more than the pages of `window` tokens and the page that the next token opens.
+  bool chunked = false;
   std::vector<int32_t> free_list;
   std::vector<uint8_t> in_use;
 };
@@ -65,14 +69,15 @@ void* cm_create(int n_groups, const int32_t* page_sizes, const int32_t* num_page
                 int n_state_slots) {
   if (n_groups < 0 || n_state_slots < 0) return nullptr;
   for (int i = 0; i < n_groups; ++i)
-    if (page_sizes[i] <= 0 || num_pages[i] < 0 || windows[i] < 0) return nullptr;
+    if (page_sizes[i] <= 0 || num_pages[i] < 0) return nullptr;
   Manager* m = new Manager();
   m->groups.resize(n_groups);
   for (int i = 0; i < n_groups; ++i) {
     Group& g = m->groups[i];
     g.page_size = page_sizes[i];
     g.num_pages = num_pages[i];
-    g.window = windows[i];
+    g.window = windows[i] < 0 ? -windows[i] : windows[i];      // (a negative entry: chunks of that many positions)
+    g.chunked = windows[i] < 0;
     g.in_use.assign(g.num_pages, 0);
     g.free_list.reserve(g.num_pages);
     // page 0 is handed out first
@@ -177,7 +182,8 @@ int cm_reserve(void* h, int64_t id, int64_t new_len) {
 }
 
 // Gives back, in windowed groups, the pages that no token at position >= computed_len can see any more:
-// a query at position p sees keys p - W + 1 .. p, so every key below computed_len - W + 1 is dead.
+// a query at position p sees keys p - W + 1 .. p, so every key below computed_len - W + 1 is dead; with chunks of W
+// positions the next token sees its chunk from (computed_len / W) * W on.
 // Returns the number of pages released.
 int cm_release_behind(void* h, int64_t id, int64_t computed_len) {
   Manager* m = static_cast<Manager*>(h);
@@ -188,7 +194,7 @@ int cm_release_behind(void* h, int64_t id, int64_t computed_len) {
   for (size_t gi = 0; gi < m->groups.size(); ++gi) {
     Group& g = m->groups[gi];
     if (g.window <= 0) continue;
-    const int64_t first_needed = computed_len - g.window + 1;
+    const int64_t first_needed = g.chunked ? (computed_len / g.window) * g.window : computed_len - g.window + 1;
     if (first_needed <= 0) continue;
     int64_t dead_blocks = first_needed / g.page_size;  // blocks wholly below first_needed
     if (dead_blocks > (int64_t)r.tables[gi].size()) dead_blocks = (int64_t)r.tables[gi].size();

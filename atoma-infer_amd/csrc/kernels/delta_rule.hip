@@ -56,9 +56,12 @@ delta_prepare_kernel(const float* __restrict__ proj, DeltaShape sh, const int32_
     return;
   }
   const float* conv_state = state + (size_t)state_slots[e] * state_stride;
+  // (unrolled so that the loads of several channels and taps are in flight together)
+#pragma unroll 4
   for (int c = threadIdx.x; c < channels; c += 256) {
     const int col = c < nqk ? sh.off_q + c : c < 2 * nqk ? sh.off_k + (c - nqk) : sh.off_v + (c - 2 * nqk);
     float y = 0.f;
+#pragma unroll 4
     for (int j = 0; j < sh.taps; ++j) {
       const int s = n - (sh.taps - 1) + j;      // index inside the entry of the input under tap j
       const float x = s >= 0 ? proj[(size_t)(t - (sh.taps - 1) + j) * sh.ldp + col]

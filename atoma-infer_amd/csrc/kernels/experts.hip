@@ -168,17 +168,20 @@ gather_scale_kernel(const uint16_t* __restrict__ x, int ldx, const float* __rest
   for (int k = threadIdx.x; k < K; k += 256) xs[(size_t)place * K + k] = f32_to_bf16_bits(bf16_bits_to_f32(src[k]) * sc);
 }
 
-constexpr int kLdsRow = 64 + 8;     // bfloat16 elements a row of the activations' tile takes in LDS (padded)
 
-// NS: blocks of 16 rows of the weight a wave takes (2 or 4: a fragment of the activations read from LDS then feeds as
-// many products, and LDS is what bounds a tile of 128 places)
-template <bool SWIGLU, int TM, int NS>
+// NS: blocks of 16 rows of the weight a wave takes.  KSUB: pieces of 32 columns of K a step (2, or 4 for tiles of 64
+// places: a decode step's tile holds a place or two, the product streams the weight, and what it needs is many bytes
+// in flight a step).
+template <bool SWIGLU, int TM, int NS, int KSUB>
 __global__ void __launch_bounds__(256)
 expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, void* __restrict__ c, int ldc,
                         int N, int K, const int32_t* __restrict__ perm, const int32_t* __restrict__ offsets,
                         const int32_t* __restrict__ tiles, int top, int plane_rows) {
   constexpr int MS = TM / 16;          // blocks of 16 places a tile
-  constexpr int AP = TM / 32;          // 16-byte pieces of the activations' tile a thread moves a step
+  constexpr int KSTEP = 32 * KSUB;     // columns of K a step
+  constexpr int kLdsRow = KSTEP + 8;   // bfloat16 elements a row of the activations' tile takes in LDS (padded)
+  constexpr int SEGS = KSTEP / 8;      // 16-byte pieces a row of the tile
+  constexpr int AP = TM * SEGS / 256;  // ... and a thread moves a step
   __shared__ __attribute__((aligned(16))) uint16_t at[TM * kLdsRow];
   const int e = tiles[2 * blockIdx.y];
   if (e < 0) return;
@@ -205,36 +208,36 @@ expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restri
 
   // The operands of a step are asked for a step ahead: the weight's fragments wait in registers, the activations' pieces
   // too, until the tile of the step before has been read and they may go to LDS.
-  bf16x8 wf[2][NS], wn[2][NS];
+  bf16x8 wf[KSUB][NS], wn[KSUB][NS];
   uint4 ar[AP];
-  auto fetch = [&](int k0, bf16x8 (&dst)[2][NS]) {
+  auto fetch = [&](int k0, bf16x8 (&dst)[KSUB][NS]) {
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
+    for (int kk = 0; kk < KSUB; ++kk)
 #pragma unroll
       for (int s = 0; s < NS; ++s) {
-        // (K is a multiple of 32: the last step may have its first half only)
+        // (K is a multiple of 32: the last step may be short)
         if (k0 + kk * 32 < K) dst[kk][s] = *reinterpret_cast<const bf16x8*>(wp[s] + k0 + kk * 32);
         else dst[kk][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
       }
 #pragma unroll
     for (int i = 0; i < AP; ++i) {
-      const int idx = tid + i * 256, r = idx >> 3, seg = idx & 7;
+      const int idx = tid + i * 256, r = idx / SEGS, seg = idx % SEGS;
       ar[i] = make_uint4(0, 0, 0, 0);
       if (r < rows && k0 + seg * 8 < K) ar[i] = *reinterpret_cast<const uint4*>(a + (size_t)(row0 + r) * K + k0 + seg * 8);
     }
   };
   fetch(0, wf);
-  for (int k0 = 0; k0 < K; k0 += 64) {
+  for (int k0 = 0; k0 < K; k0 += KSTEP) {
     __syncthreads();          // the tile of the step before has been read
 #pragma unroll
     for (int i = 0; i < AP; ++i) {
-      const int idx = tid + i * 256, r = idx >> 3, seg = idx & 7;
+      const int idx = tid + i * 256, r = idx / SEGS, seg = idx % SEGS;
       if (r < msub * 16) *reinterpret_cast<uint4*>(at + r * kLdsRow + seg * 8) = ar[i];
     }
     __syncthreads();
-    if (k0 + 64 < K) fetch(k0 + 64, wn);
+    if (k0 + KSTEP < K) fetch(k0 + KSTEP, wn);
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
+    for (int kk = 0; kk < KSUB; ++kk) {
 #pragma unroll
       for (int m = 0; m < MS; ++m) {
         if (m < msub) {
@@ -246,7 +249,7 @@ expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restri
       }
     }
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
+    for (int kk = 0; kk < KSUB; ++kk)
 #pragma unroll
       for (int s = 0; s < NS; ++s) wf[kk][s] = wn[kk][s];
   }
@@ -305,13 +308,13 @@ extern "C" int atoma_expert_gemm_mfma(const void* a, const void* w, void* c, int
     return ATOMA_ERR_SHAPE;
   const int ns = 2;      // (four blocks a wave measured slower for tiles of 128 places: 467 against 336 us)
   dim3 grid((N + 64 * ns - 1) / (64 * ns), max_tiles), block(256);
-#define ATOMA_EGM(SW, TM_, NS_)                                                                                  \
-  hipLaunchKernelGGL((expert_gemm_mfma_kernel<SW, TM_, NS_>), grid, block, 0, stream, (const uint16_t*)a,        \
+#define ATOMA_EGM(SW, TM_, NS_, KSUB_)                                                                           \
+  hipLaunchKernelGGL((expert_gemm_mfma_kernel<SW, TM_, NS_, KSUB_>), grid, block, 0, stream, (const uint16_t*)a, \
                      (const uint16_t*)w, c, ldc, N, K, perm, offsets, tiles, top, plane_rows)
-  if (swiglu && tile_m == 64) ATOMA_EGM(true, 64, 2);
-  else if (swiglu) ATOMA_EGM(true, 128, 2);
-  else if (tile_m == 64) ATOMA_EGM(false, 64, 2);
-  else ATOMA_EGM(false, 128, 2);
+  if (swiglu && tile_m == 64) ATOMA_EGM(true, 64, 2, 4);
+  else if (swiglu) ATOMA_EGM(true, 128, 2, 2);
+  else if (tile_m == 64) ATOMA_EGM(false, 64, 2, 4);
+  else ATOMA_EGM(false, 128, 2, 2);
 #undef ATOMA_EGM
   ATOMA_LAUNCH_CHECK();
   return 0;

@@ -65,7 +65,7 @@ class PagedAttention(Mixer):
                 "v_proj.weight": WeightSpec((kv, self.width)), "o_proj.weight": WeightSpec((self.width, q))}
 
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec(self.nkv, self.hd, self.window)
+        return CacheSpec(self.nkv, self.hd, self.window, chunk=self.chunk)
 
     def load(self, get, device, act_dtype) -> None:
         ws = [get("q_proj.weight"), get("k_proj.weight"), get("v_proj.weight")]

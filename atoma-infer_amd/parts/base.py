@@ -55,8 +55,9 @@ class WeightSpec:
 class CacheSpec:
     """What a mixer keeps per token: keys and values of ``kv_heads`` heads of ``head_size``.
 
-    ``window``: None keeps every token; w keeps the last w.  Layers whose specs are equal share one
-    group of pages and one block table per request.
+    ``window``: None keeps every token; w keeps the last w.  ``chunk``: c keeps the tokens of the current chunk of c
+    positions (chunks count from the request's first position), for mixers whose tokens see their own chunk only.
+    Layers whose specs are equal share one group of pages and one block table per request.
 
     ``value_size``: elements per head and token of the second tensor, when it is not as wide as the first: None
     means ``head_size``; 0 means that the mixer keeps one tensor only (a latent vector per token, say) and its
@@ -67,9 +68,11 @@ class CacheSpec:
     head_size: int
     window: Optional[int] = None
     value_size: Optional[int] = None
+    chunk: Optional[int] = None
 
     def __post_init__(self):
-        if self.kv_heads <= 0 or self.head_size <= 0 or (self.value_size is not None and self.value_size < 0):
+        if self.kv_heads <= 0 or self.head_size <= 0 or (self.value_size is not None and self.value_size < 0) \
+                or (self.window and self.chunk):
             raise ValueError(f"invalid cache spec: {self}")
 
     @property

@@ -222,7 +222,7 @@ def compare_main(args) -> int:
     from atoma_infer_amd.models import random_model
     sizes = args.sizes if args.sizes in ("1b", "3b") else "1b"
     layers = args.layers or 4
-    llama = dict(LLAMA_1B, **OTHER_SIZES.get(sizes, {}), num_hidden_layers=layers)
+    llama = dict(dict(LLAMA_1B, **OTHER_SIZES.get(sizes, {})), num_hidden_layers=layers)
     sun = somesun_like(llama, layers)
     out = {}
     for name, cfg in (("llama", llama), ("somesun", sun)):

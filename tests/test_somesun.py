@@ -202,3 +202,23 @@ def test_plain_experts_weigh_the_input_not_the_output():
 
 def test_plain_layer_without_a_feed_forward_and_layer_helper():
     assert layer(left=dict(dim=8))["mixer"]["left"]["dim"] == 8 and layer(mlp=None)["mlp"] is None
+
+
+def test_pages_behind_a_token_s_chunk_go_back_while_the_request_runs():
+    from atoma_infer_amd.cache.manager import CacheManager, GroupGeometry
+    m = CacheManager([GroupGeometry(16, 12, None, 40)], 2)
+    m.add(7)
+    m.reserve(7, 100)
+    assert m.table(7) == [0, 1, 2, 3, 4, 5, 6]
+    # the token at position 100 sees keys 80 .. 100: the five pages wholly below 80 are dead
+    assert m.release_behind(7, 100) == 5 and m.table(7) == [-1] * 5 + [5, 6]
+    assert m.release_behind(7, 119) == 0             # still in the chunk that began at 80
+    m.reserve(7, 121)
+    # position 120 opens a chunk in the middle of a page, which stays; the pages before it go
+    assert m.release_behind(7, 120) == 2 and m.table(7)[:7] == [-1] * 7 and m.table(7)[7] >= 0
+    m.check()
+    m.free(7)
+    m.check()
+    assert m.num_free_pages() == 12
+    _, _, spec = build(SUN_A)
+    assert [g.spec.chunk for g in plan_cache(spec).groups] == [7, 16]
