@@ -246,6 +246,42 @@ delta_out_kernel(const float* __restrict__ o, const float* __restrict__ gate_pre
   }
 }
 
+// The second half of a low-rank map for few tokens: out[t, n] = sum_k x[t, k] * w[n, k], K small (the inner size of
+// the map), float32 sums in ascending order of k.  A thread an output; the token's K inputs wait in LDS.  With many
+// tokens the general product is the better kernel (it reads a tile of w once for 64 tokens).
+template <typename TW>
+__global__ void __launch_bounds__(256)
+lowrank_up_kernel(const float* __restrict__ x, int ldx, const TW* __restrict__ w, float* __restrict__ out, int ldo,
+                  int N, int K) {
+  extern __shared__ float xs[];
+  const int t = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x;
+  for (int k = threadIdx.x; k < K; k += 256) xs[k] = x[(size_t)t * ldx + k];
+  __syncthreads();
+  if (n >= N) return;
+  const TW* wr = w + (size_t)n * K;
+  float acc = 0.f;
+#pragma unroll 8
+  for (int k = 0; k < K; ++k) acc = fmaf(xs[k], to_f32(wr[k]), acc);
+  out[(size_t)t * ldo + n] = acc;
+}
+
+extern "C" int atoma_lowrank_up(const float* x, int ldx, const void* w, int w_dtype, float* out, int ldo, int n_tokens,
+                                int N, int K, hipStream_t stream) {
+  if (n_tokens <= 0 || N <= 0) return 0;
+  if (K <= 0 || K > 8192 || ldx < K || ldo < N || n_tokens > 65535) return ATOMA_ERR_SHAPE;
+  dim3 grid((N + 255) / 256, n_tokens), block(256);
+  if (w_dtype == kBF16)
+    hipLaunchKernelGGL((lowrank_up_kernel<bf16_t>), grid, block, K * sizeof(float), stream, x, ldx, (const bf16_t*)w,
+                       out, ldo, N, K);
+  else if (w_dtype == kF32)
+    hipLaunchKernelGGL((lowrank_up_kernel<float>), grid, block, K * sizeof(float), stream, x, ldx, (const float*)w, out,
+                       ldo, N, K);
+  else
+    return ATOMA_ERR_DTYPE;
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
 static bool shape_ok(const DeltaShape& sh) {
   return sh.heads > 0 && sh.kv_heads > 0 && sh.heads % sh.kv_heads == 0 && sh.dim > 0 && sh.dim <= 256 && sh.vdim > 0 &&
          sh.taps >= 1 && sh.taps <= 64 && sh.ldp > 0;

@@ -329,11 +329,13 @@ def add_normed(resid: torch.Tensor, terms, w_post: torch.Tensor, eps_post: float
 def qk_norm_rope(qk: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, rot_dim: int, wq: torch.Tensor,
                  wk: torch.Tensor, eps: float, q_out: torch.Tensor, kcache: Optional[torch.Tensor],
                  vcache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor], page_size: int, nh: int,
-                 nkv: int, hd: int) -> None:
+                 nkv: int, hd: int, hd_out: Optional[int] = None) -> None:
     """From qk float32 [T, >= (nh + nkv) hd]: q and k normed over their whole projections (weights wq [nh hd],
     wk [nkv hd]), the first ``rot_dim`` columns of every head rotated in neighbouring pairs by position *
     inv_freq[i]; q to ``q_out`` [T, nh hd], k into ``kcache`` tiles at ``slot_mapping``; ``vcache`` (optional)
-    receives the k projection as it came."""
+    receives the k projection as it came.  ``hd_out`` > hd: heads leave ``hd_out`` wide, zeros beyond hd, in
+    ``q_out`` [T, nh hd_out] and in the tiles."""
+    hd_out = hd if hd_out is None else int(hd_out)
     _dev(qk, positions, inv_freq, wq, wk, q_out, kcache, vcache, slot_mapping)
     t = qk.shape[0]
     _need(qk.dtype is torch.float32 and qk.dim() == 2 and qk.stride(1) == 1 and qk.shape[1] >= (nh + nkv) * hd,
@@ -342,14 +344,14 @@ def qk_norm_rope(qk: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tens
     _f32(inv_freq, "inv_freq", rot_dim // 2)
     _f32(wq, "q norm weight", nh * hd)
     _f32(wk, "k norm weight", nkv * hd)
-    _need(q_out.dim() == 2 and q_out.stride(1) == 1 and q_out.shape[0] == t and q_out.shape[1] >= nh * hd,
-          "q_out must be [T, nh hd]")
+    _need(hd_out >= hd and q_out.dim() == 2 and q_out.stride(1) == 1 and q_out.shape[0] == t
+          and q_out.shape[1] >= nh * hd_out, "q_out must be [T, nh hd_out]")
     cache_code = _code(q_out, "q_out")
     if kcache is not None:
         _need(slot_mapping is not None, "a cache write needs slots")
         _i32(slot_mapping, "slot_mapping", t)
         pages = kcache.shape[0]
-        _need(kcache.is_contiguous() and tuple(kcache.shape) == (pages, nkv, page_size * hd), "key tiles: bad shape")
+        _need(kcache.is_contiguous() and tuple(kcache.shape) == (pages, nkv, page_size * hd_out), "key tiles: bad shape")
         cache_code = _code(kcache, "cache")
         if vcache is not None:
             _need(vcache.is_contiguous() and tuple(vcache.shape) == tuple(kcache.shape)
@@ -359,7 +361,7 @@ def qk_norm_rope(qk: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tens
     _check(_module("layer_norms").atoma_qk_norm_rope(
         _p(qk), qk.stride(0), _p(positions), _p(inv_freq), int(rot_dim), _p(wq), _p(wk), ctypes.c_float(eps),
         _p(q_out), q_out.stride(0), _code(q_out, "q_out"), _p(kcache), _p(vcache), cache_code, _p(slot_mapping),
-        int(page_size), t, nh, nkv, hd, _stream()), "qk_norm_rope")
+        int(page_size), t, nh, nkv, hd, hd_out, _stream()), "qk_norm_rope")
 
 
 def delta_prepare(proj: torch.Tensor, offsets, heads: int, kv_heads: int, dim: int, vdim: int, taps: int,
@@ -399,6 +401,23 @@ def delta_prepare(proj: torch.Tensor, offsets, heads: int, kv_heads: int, dim: i
         dt_pre.stride(0) if t > 1 else nd, _p(dt_bias),
         _p(a_log), _p(qn), _p(kn), _p(vn), _p(beta), _p(decay), _p(kq), t, s, _stream()), "delta_prepare")
     return qn, kn, vn, beta, decay, kq
+
+
+LOWRANK_UP_MAX_TOKENS = 32      # beyond, the general product reads a tile of the weight once for 64 tokens
+
+
+def lowrank_up(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """x float32 [T, K] (row stride free) times w [N, K] transposed, float32 out, for few tokens and a small K: the
+    second half of a low-rank map (float32 multiply-adds in ascending order of k, as the general product's)."""
+    _dev(x, w)
+    t, k = x.shape
+    n = w.shape[0]
+    _need(x.dtype is torch.float32 and x.stride(1) == 1 and w.dim() == 2 and w.is_contiguous() and w.shape[1] == k,
+          "lowrank_up: operands do not fit")
+    out = torch.empty((t, n), dtype=torch.float32, device=x.device)
+    _check(_module("delta_rule").atoma_lowrank_up(_p(x), x.stride(0) if t > 1 else k, _p(w), _code(w, "w"), _p(out), n,
+                                                  t, n, k, _stream()), "lowrank_up")
+    return out
 
 
 def delta_scan(qn, kn, vn, beta, decay, kq, heads: int, kv_heads: int, dim: int, vdim: int, taps: int,

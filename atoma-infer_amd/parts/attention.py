@@ -198,7 +198,10 @@ class TiedValueAttention(PagedAttention):
       [heads * head_size] and ``k.norm`` [kv_heads * head_size], before the rotation;
     * the first ``rotary_dim`` columns of every head are rotated in neighbouring pairs (2i, 2i + 1) by
       position * base^(-2i / rotary_dim), angles in float32, for any position (no table);
-    * optional chunks and one learned sink per head (tensor ``sink``), see ``PagedAttention``.
+    * optional chunks and one learned sink per head (tensor ``sink``), see ``PagedAttention``;
+    * any even head size up to 256: one that is no multiple of 16 runs as the next multiple of 16, with zeros in the
+      added columns of the queries, of both tiles of the cache and of the output projection (``self.hd`` is the
+      size the cache and the attention kernels see, ``self.hd_in`` the checkpoint's).
 
     Tensors: ``q``, ``k``, ``o`` ([out, in]), ``q.norm``, ``k.norm``, ``sink``.
     """
@@ -206,7 +209,9 @@ class TiedValueAttention(PagedAttention):
     def __init__(self, width: int, num_heads: int, num_kv_heads: int, head_size: int, scale: float, norm_eps: float,
                  rotary_base: float, rotary_dim: int, chunk: Optional[int] = None, window: Optional[int] = None,
                  sink: bool = True):
-        super().__init__(width, num_heads, num_kv_heads, head_size, None, window, scale, chunk)
+        self.hd_in = int(head_size)
+        padded = -(-self.hd_in // 16) * 16      # (multiples of 16: what the matrix-core kernel takes)
+        super().__init__(width, num_heads, num_kv_heads, padded, None, window, scale, chunk)
         if head_size % 2 or rotary_dim % 2 or not 0 <= rotary_dim <= head_size or rotary_dim > 256:
             raise ValueError(f"rotary_dim {rotary_dim} must be even, at most the head size {head_size} and at most 256")
         self.norm_eps, self.rotary_base, self.rotary_dim, self.has_sink = float(norm_eps), float(rotary_base), \
@@ -217,7 +222,7 @@ class TiedValueAttention(PagedAttention):
         return True
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        q, kv = self.nh * self.hd, self.nkv * self.hd
+        q, kv = self.nh * self.hd_in, self.nkv * self.hd_in
         specs = {"q": WeightSpec((q, self.width)), "k": WeightSpec((kv, self.width)),
                  "q.norm": WeightSpec((q,), "norm"), "k.norm": WeightSpec((kv,), "norm"),
                  "o": WeightSpec((self.width, q))}
@@ -229,7 +234,10 @@ class TiedValueAttention(PagedAttention):
         ws = [get("q"), get("k")]
         dt = ws[0].dtype if ws[0].dtype is ws[1].dtype else torch.float32
         self.w_qk = torch.cat([w.to(device=device, dtype=dt) for w in ws], dim=0).contiguous()
-        self.w_o = get("o").to(device).contiguous()
+        w_o = get("o").to(device)
+        if self.hd != self.hd_in:      # zero columns under the heads' added columns
+            w_o = torch.nn.functional.pad(w_o.view(self.width, self.nh, self.hd_in), (0, self.hd - self.hd_in))
+        self.w_o = w_o.reshape(self.width, self.nh * self.hd).contiguous()
         f32 = dict(device=device, dtype=torch.float32)
         self.q_norm, self.k_norm = get("q.norm").to(**f32).contiguous(), get("k.norm").to(**f32).contiguous()
         self.sinks = get("sink").to(**f32).contiguous() if self.has_sink else None
@@ -260,7 +268,7 @@ class TiedValueAttention(PagedAttention):
         qk = linear(x, w, torch.float32)
         q = torch.empty((t, nh * hd), dtype=x.dtype, device=x.device)
         ops.qk_norm_rope(qk, ctx.positions, self.inv_freq, self.rotary_dim, self.q_norm, self.k_norm, self.norm_eps, q,
-                         cache.k, cache.v, cache.slot_mapping, cache.page_size, nh, nkv, hd)
+                         cache.k, cache.v, cache.slot_mapping, cache.page_size, nh, nkv, self.hd_in, hd)
         out = torch.empty((t, nh * hd), dtype=x.dtype, device=x.device)
         self.attend(q, cache.k, cache.v, out, ctx, cache)
         return linear_delta(out, self.w_o, None, self.w_o_tiled)

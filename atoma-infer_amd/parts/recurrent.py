@@ -114,7 +114,9 @@ class GatedDeltaRule(Mixer):
         state = cache.state
         proj = linear(x, self.w_in, torch.float32)
         # the second halves of the two low-rank maps read their columns of the float32 projection as they are
-        pre = linear(proj[:, self.off_a1: self.off_g1 + self.gate_rank], self.w_ag, torch.float32)
+        low = proj[:, self.off_a1: self.off_g1 + self.gate_rank]
+        pre = ops.lowrank_up(low, self.w_ag) if x.shape[0] <= ops.LOWRANK_UP_MAX_TOKENS else \
+            linear(low, self.w_ag, torch.float32)
         dt_pre, gate_pre = pre[:, : self.nd], pre[:, self.nd:]
         qn, kn, vn, beta, decay, kq = ops.delta_prepare(
             proj, (self.off_q, self.off_k, self.off_v, self.off_b), self.heads, self.kv_heads, self.dim, self.vdim,

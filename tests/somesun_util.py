@@ -49,6 +49,13 @@ SUN_B = config([
           right={"dim": 128, "heads": 2, "kv_heads": 2, "vdim": 16, "conv": 1},
           mlp={"ff": 32, "experts": 5, "top": 3}),
 ], width=128, vocab=211, eps=3e-6)
+# head sizes that the matrix-core attention does not take as they are (36 and 40: run as 48)
+SUN_C = config([
+    layer(left={"dim": 36, "heads": 2, "kv_heads": 1, "scale": 0.2, "mask": {"size": 11}, "rot": {"base": 77.0, "dims": 18}},
+          right={"dim": 24, "heads": 2, "kv_heads": 1, "vdim": 12, "conv": 2}, mlp={"ff": 32, "experts": 2, "top": 2}),
+    layer(left={"dim": 40, "heads": 3, "kv_heads": 3, "scale": 0.15, "mask": {"size": 64}, "rot": {"base": 77.0, "dims": 40}},
+          right={"dim": 8, "heads": 1, "kv_heads": 1, "vdim": 64, "conv": 3}, mlp={"ff": 40, "experts": 6, "top": 1}),
+], width=96, vocab=130)
 
 
 def write_model(path: str, cfg: dict, seed: int, changes=None) -> str:

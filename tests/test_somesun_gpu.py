@@ -7,7 +7,7 @@ import pytest
 import torch
 
 import plain_somesun as ps
-from somesun_util import (SUN_A, SUN_B, TOL, assert_logits, config, layer, logit_err, make_runner, plain_config, plain_weights,
+from somesun_util import (SUN_A, SUN_B, SUN_C, TOL, assert_logits, config, layer, logit_err, make_runner, plain_config, plain_weights,
                           run_schedule, tokens, write_model)
 
 pytestmark = pytest.mark.gpu
@@ -17,7 +17,8 @@ DEV = "cuda:0"
 @pytest.fixture(scope="module")
 def dirs(tmp_path_factory):
     root = tmp_path_factory.mktemp("somesun")
-    return {"A": write_model(str(root / "a"), SUN_A, 11), "B": write_model(str(root / "b"), SUN_B, 12)}
+    return {"A": write_model(str(root / "a"), SUN_A, 11), "B": write_model(str(root / "b"), SUN_B, 12),
+            "C": write_model(str(root / "c"), SUN_C, 13)}
 
 
 def oracle(path, toks):
@@ -194,7 +195,7 @@ def _attention_case(dtype, hd, nh, nkv, chunk, rot, lens_and_cuts, page, sink_va
     tables = [[order.pop() for _ in range(-(-n // page))] for n in lens]
     max_blocks = max(len(tb) for tb in tables)
     cdt = dtype
-    k = torch.zeros((n_pages, nkv, page * hd), dtype=cdt, device=DEV)
+    k = torch.zeros((n_pages, nkv, page * part.hd), dtype=cdt, device=DEV)      # (part.hd: the size the kernels see)
     v = torch.zeros_like(k)
     got, at = [[], []], [0, 0]
     for cuts in lens_and_cuts:
@@ -219,8 +220,11 @@ CUTS = [[(0, 20), (1, 3)], [(0, 1), (1, 1)], [(0, 2)], [(1, 40), (0, 1)], [(0, 5
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("hd, nh, nkv, chunk, rot, page", [(32, 4, 2, 7, 16, 16), (64, 8, 2, 33, 64, 16), (48, 2, 1, 16, 48, 32),
-                                                           (64, 4, 4, 1, 0, 16), (24, 3, 1, 1000, 24, 4)])
+                                                           (64, 4, 4, 1, 0, 16), (24, 3, 1, 1000, 24, 4),
+                                                           (20, 3, 1, 9, 10, 16), (36, 2, 2, 50, 36, 32)])
 def test_tied_value_attention_alone(hd, nh, nkv, chunk, rot, page, dtype):
+    """Head sizes that are multiples of 16 and others (run as the next multiple of 16, zeros in the added columns); chunks of one position and chunks longer
+    than the requests; no column rotated, some, all; pages of 4, 16 and 32 tokens."""
     got, want = _attention_case(dtype, hd, nh, nkv, chunk, rot, CUTS, page)
     for a, b in zip(got, want):
         err = (a.double() - b).norm() / b.norm()
@@ -271,7 +275,7 @@ def test_sinks_and_chunks_where_a_token_s_keys_are_cut_into_parts(monkeypatch, s
 # ---- the whole model through the step function --------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_whole_prompts_token_by_token_decoding_and_portions(dirs, name, dtype):
     d = dirs[name]
     vocab = plain_config(d)["vocab"]
