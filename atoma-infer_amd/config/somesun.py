@@ -14,7 +14,7 @@ from __future__ import annotations
 import dataclasses
 from typing import Any, Dict, Optional, Tuple
 
-from .base import ConfigError, ModelConfig, as_float, as_positive_int, key, optional, parse_fields
+from .base import ConfigError, ModelConfig, as_float, as_int, as_positive_int, key, optional, parse_fields
 
 
 def _obj(cls, where: str):
@@ -35,13 +35,13 @@ class ChunkMask:
 @dataclasses.dataclass(frozen=True)
 class PairRotation:
     base: float = key(convert=as_float)
-    dims: int = key(convert=as_positive_int)
+    dims: int = key(convert=as_int)       # 0: nothing is rotated
 
     @classmethod
     def from_json(cls, obj, where="rot"):
         r = cls(**parse_fields(cls, obj, where))
-        if r.dims % 2 or not r.base > 0:
-            raise ConfigError(f"{where}: dims must be even and base positive")
+        if r.dims < 0 or r.dims % 2 or not r.base > 0:
+            raise ConfigError(f"{where}: dims must be even and not negative, base positive")
         return r
 
 

@@ -332,6 +332,34 @@ def test_decode_steps_replayed_as_graphs_give_the_eager_logits(dirs):
         assert_logits(got[i], want[i], "bfloat16", i)
 
 
+def test_a_lone_prompt_s_step_replayed_as_a_graph(dirs):
+    """A step that is one prompt of 256 tokens or more and wants its last place is recorded the third time its shape is
+    seen: every replay, with other tokens and another state slot, gives what a runner without graphs gives."""
+    from atoma_infer_amd.engine.step import StepEntry
+    d = dirs["B"]
+    vocab = plain_config(d)["vocab"]
+    runner = make_runner(d, "bfloat16", 1024, 16, 4)
+    eager = make_runner(d, "bfloat16", 1024, 16, 4)
+    eager.use_graphs = False
+    n = 300
+    for r in (runner, eager):         # holds a slot and pages throughout, so the prompts below get other ones in turn
+        r.add_request(100)
+        r.step([StepEntry(100, tokens(20, vocab, 1), 0, [19])])
+    for i in range(5):
+        toks = tokens(n + 1, vocab, 70 + i)
+        got = []
+        for r in (runner, eager):
+            r.add_request(i)
+            a = r.step([StepEntry(i, toks[:n], 0, [n - 1])]).float().cpu().clone()
+            b = r.step([StepEntry(i, toks[n:], n, [0])]).float().cpu().clone()
+            if i < 4:
+                r.free_request(i)
+            got.append(torch.cat([a, b]))
+        assert logit_err(got[0], got[1]) < 1e-3, (i, logit_err(got[0], got[1]))
+    assert any(isinstance(k, tuple) and k[0] == "prompt" and g.graph is not None for k, g in runner._graphs.items())
+    assert not eager._graphs
+
+
 def test_decoding_with_a_token_s_keys_cut_into_parts(dirs, monkeypatch):
     """The same with the attention kernel made to cut the keys of decoded tokens into parts, as it does by itself only
     at contexts and chunk sizes beyond those of a quick test."""
