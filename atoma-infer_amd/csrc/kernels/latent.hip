@@ -1,0 +1,124 @@
+// Attention over one small cached vector per token: the kernels around the paged attention kernels.
+//
+// A token's keys and values of every head are products of one latent vector c (rank numbers), so the cache holds c
+// alone and the heads' key and value maps move to the query's side:
+//
+//   score_h(i, j) = (W_uk,h c_j) . q_h,i = c_j . (W_uk,h^T q_h,i),       out_h,i = W_uv,h (sum_j p_ij c_j),
+//
+// which is attention with one shared key/value head of `rank` columns whose values are its keys.
+//   latent_prepare   per token: c = rmsnorm(down projection) * w into the cache (as key and as value: the two tiles
+//                    differ in the order of their elements only), the heads' gates sigmoid(g) in float32, and q in
+//                    the activation dtype;
+//   head_linear      per head a product of its own: out[t, h, :] = W[h] x[t, h, :], optionally times a scalar per
+//                    (token, head), float32 sums in an order that depends on the sizes alone.
+#include "common.h"
+#include "cache_layout.h"
+
+using namespace atoma;
+
+// proj [T, ldp] float32: q (heads * dim columns from off_q), the down projection (rank from off_c), gates (heads from
+// off_g).  Cache tiles hold rank_p >= rank columns a token; the added ones are zero.
+template <typename TA, typename TC>
+__global__ void __launch_bounds__(256)
+latent_prepare_kernel(const float* __restrict__ proj, int ldp, int off_q, int off_c, int off_g, int nq, int rank,
+                      int rank_p, int heads, const float* __restrict__ w_norm, float eps,
+                      TC* __restrict__ kcache, TC* __restrict__ vcache, const int32_t* __restrict__ slot_mapping,
+                      int page_size, TA* __restrict__ q_out, float* __restrict__ gate) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x;
+  const float* row = proj + (size_t)t * ldp;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < rank; i += 256) ss = fmaf(row[off_c + i], row[off_c + i], ss);
+  ss = block_sum<4>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)rank + eps);
+  const int slot = slot_mapping[t];
+  if (slot >= 0) {
+    const int page = slot / page_size, off = slot % page_size;
+    TC* ktile = kcache + (size_t)page * page_size * rank_p;
+    TC* vtile = vcache + (size_t)page * page_size * rank_p;
+    for (int i = threadIdx.x; i < rank_p; i += 256) {
+      const TC c = from_f32<TC>(i < rank ? row[off_c + i] * inv * w_norm[i] : 0.f);
+      ktile[key_offset(off, i, page_size)] = c;
+      vtile[value_offset(i, off, rank_p, page_size)] = c;
+    }
+  }
+  for (int i = threadIdx.x; i < nq; i += 256) q_out[(size_t)t * nq + i] = from_f32<TA>(row[off_q + i]);
+  for (int h = threadIdx.x; h < heads; h += 256) gate[(size_t)t * heads + h] = 1.0f / (1.0f + expf(-row[off_g + h]));
+}
+
+// out[t, h * N + n] = (sum_k x[t, h * K + k] * w[(h * N + n) * K + k]) * (gate ? gate[t * H + h] : 1)
+// A workgroup: 16 tokens x 64 outputs of one head; K in chunks of 32 through LDS.
+template <typename TA, typename TW, typename TO>
+__global__ void __launch_bounds__(256)
+head_linear_kernel(const TA* __restrict__ x, int ldx, const TW* __restrict__ w, TO* __restrict__ out, int ldo,
+                   const float* __restrict__ gate, int T, int H, int K, int N) {
+  __shared__ float xs[16][33], ws[64][33];
+  const int h = blockIdx.z, n0 = blockIdx.x * 64, t0 = blockIdx.y * 16;
+  const int nl = threadIdx.x & 63, rg = threadIdx.x >> 6;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 16 * 32; idx += 256) {
+      const int r = idx >> 5, kk = idx & 31;
+      xs[r][kk] = (t0 + r < T && k0 + kk < K) ? to_f32(x[(size_t)(t0 + r) * ldx + (size_t)h * K + k0 + kk]) : 0.f;
+    }
+    for (int idx = threadIdx.x; idx < 64 * 32; idx += 256) {
+      const int r = idx >> 5, kk = idx & 31;
+      ws[r][kk] = (n0 + r < N && k0 + kk < K) ? to_f32(w[((size_t)h * N + n0 + r) * K + k0 + kk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 32; ++kk) {
+      const float wv = ws[nl][kk];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = fmaf(xs[rg + 4 * i][kk], wv, acc[i]);
+    }
+  }
+  if (n0 + nl >= N) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = t0 + rg + 4 * i;
+    if (t < T) {
+      const float s = gate ? gate[(size_t)t * H + h] : 1.0f;
+      out[(size_t)t * ldo + (size_t)h * N + n0 + nl] = from_f32<TO>(acc[i] * s);
+    }
+  }
+}
+
+extern "C" int atoma_latent_prepare(const float* proj, int ldp, int off_q, int off_c, int off_g, int nq, int rank,
+                                    int rank_p, int heads, const float* w_norm, float eps, void* kcache, void* vcache,
+                                    int cache_dtype, const int32_t* slot_mapping, int page_size, void* q_out,
+                                    int act_dtype, float* gate, int n_tokens, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (rank <= 0 || rank_p < rank || heads <= 0 || nq <= 0 || page_size <= 0 || ldp <= 0) return ATOMA_ERR_SHAPE;
+  dim3 grid(n_tokens), block(256);
+#define ATOMA_LATENT(TA, TC)                                                                                      \
+  hipLaunchKernelGGL((latent_prepare_kernel<TA, TC>), grid, block, 0, stream, proj, ldp, off_q, off_c, off_g, nq, \
+                     rank, rank_p, heads, w_norm, eps, (TC*)kcache, (TC*)vcache, slot_mapping, page_size,         \
+                     (TA*)q_out, gate)
+  if (act_dtype == kF32 && cache_dtype == kF32) ATOMA_LATENT(float, float);
+  else if (act_dtype == kBF16 && cache_dtype == kBF16) ATOMA_LATENT(bf16_t, bf16_t);
+  else return ATOMA_ERR_DTYPE;
+#undef ATOMA_LATENT
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int atoma_head_linear(const void* x, int x_dtype, int ldx, const void* w, int w_dtype, void* out,
+                                 int out_dtype, int ldo, const float* gate, int T, int H, int K, int N,
+                                 hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H <= 0 || K <= 0 || N <= 0 || ldx < H * K || ldo < H * N || H > 65535 || (T + 15) / 16 > 65535) return ATOMA_ERR_SHAPE;
+  dim3 grid((N + 63) / 64, (T + 15) / 16, H), block(256);
+#define ATOMA_HL(TA, TW, TO)                                                                                  \
+  hipLaunchKernelGGL((head_linear_kernel<TA, TW, TO>), grid, block, 0, stream, (const TA*)x, ldx, (const TW*)w, \
+                     (TO*)out, ldo, gate, T, H, K, N)
+  if (x_dtype == kF32 && w_dtype == kF32 && out_dtype == kF32) ATOMA_HL(float, float, float);
+  else if (x_dtype == kF32 && w_dtype == kBF16 && out_dtype == kF32) ATOMA_HL(float, bf16_t, float);
+  else if (x_dtype == kBF16 && w_dtype == kBF16 && out_dtype == kBF16) ATOMA_HL(bf16_t, bf16_t, bf16_t);
+  else if (x_dtype == kBF16 && w_dtype == kBF16 && out_dtype == kF32) ATOMA_HL(bf16_t, bf16_t, float);
+  else return ATOMA_ERR_DTYPE;
+#undef ATOMA_HL
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}

@@ -5,6 +5,9 @@
 //   resid += d / sqrt(mean(d^2) + eps) * w_post                   (float32, in place)
 //   out   = resid / sqrt(mean(resid^2) + eps) * w_next            (optional, in the activation dtype)
 //
+// Without w_post the sum joins the stream as it is, resid += d: blocks whose sublayers read one norm and add their
+// outputs side by side.
+//
 // One workgroup a row; the row waits in LDS between the passes, so every operand is read once.  All statistics and
 // sums are float32.  The planes of a term are added in the order of their index and the terms in theirs, so a row's
 // result does not depend on its place in the batch.
@@ -46,11 +49,14 @@ add_normed_kernel(float* __restrict__ resid, Term a, Term b, int n_terms, const 
     row[i] = d;
     ss += d * d;
   }
-  ss = block_sum<4>(ss, scratch);
-  const float inv = 1.0f / sqrtf(ss / (float)width + eps_post);
+  float inv = 1.0f;
+  if (w_post != nullptr) {
+    ss = block_sum<4>(ss, scratch);
+    inv = 1.0f / sqrtf(ss / (float)width + eps_post);
+  }
   float ss2 = 0.f;
   for (int i = threadIdx.x; i < width; i += 256) {
-    const float x = resid[base + i] + row[i] * inv * w_post[i];
+    const float x = resid[base + i] + (w_post != nullptr ? row[i] * inv * w_post[i] : row[i]);
     resid[base + i] = x;
     row[i] = x;
     ss2 += x * x;
@@ -148,17 +154,20 @@ add_normed_vec_kernel(float* __restrict__ resid, Term a, Term b, int n_terms, co
     if (threadIdx.x + j * 256 < n4)
 #pragma unroll
       for (int i = 0; i < 4; ++i) ss += d[j].v[i] * d[j].v[i];
-  ss = block_sum<4>(ss, scratch);
-  const float inv = 1.0f / sqrtf(ss / (float)width + eps_post);
+  float inv = 1.0f;
+  if (w_post != nullptr) {
+    ss = block_sum<4>(ss, scratch);
+    inv = 1.0f / sqrtf(ss / (float)width + eps_post);
+  }
   float ss2 = 0.f;
 #pragma unroll
   for (int j = 0; j < MAXJ; ++j) {
     const int c = threadIdx.x + j * 256;
     if (c < n4) {
-      const f4 wp = load4(w_post + 4 * c);
+      const f4 wp = w_post != nullptr ? load4(w_post + 4 * c) : f4{{1.f, 1.f, 1.f, 1.f}};
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        x[j].v[i] += d[j].v[i] * inv * wp.v[i];
+        x[j].v[i] += w_post != nullptr ? d[j].v[i] * inv * wp.v[i] : d[j].v[i];
         ss2 += x[j].v[i] * x[j].v[i];
       }
       store4(resid + base + 4 * c, x[j]);
@@ -220,6 +229,49 @@ extern "C" int atoma_add_normed(float* resid, const void* d0, int dtype0, int pl
   else if (out_dtype == kBF16)
     hipLaunchKernelGGL((add_normed_kernel<bf16_t>), grid, block, lds, stream, resid, a, b, n_terms, w_post, w_next,
                        (bf16_t*)out, width, eps_post, eps_next);
+  else
+    return ATOMA_ERR_DTYPE;
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+// Rows of the stream set anew: resid[t] = y[t] + bias (float32), for a map of the whole stream that replaces it
+// (the entry of a pass over looped layers).  The second kernel packs the rows of two float32 streams side by side in
+// the activation dtype, [a | b], as such a map's input.
+__global__ void __launch_bounds__(256)
+set_rows_kernel(float* __restrict__ resid, const float* __restrict__ y, const float* __restrict__ bias, int width) {
+  const size_t base = (size_t)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += 256) resid[base + i] = y[base + i] + bias[i];
+}
+
+template <typename TO>
+__global__ void __launch_bounds__(256)
+pack_pair_kernel(const float* __restrict__ a, const float* __restrict__ b, TO* __restrict__ out, int width) {
+  const size_t base = (size_t)blockIdx.x * width;
+  TO* o = out + 2 * base;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    o[i] = from_f32<TO>(a[base + i]);
+    o[width + i] = from_f32<TO>(b[base + i]);
+  }
+}
+
+extern "C" int atoma_set_rows(float* resid, const float* y, const float* bias, int n_rows, int width,
+                              hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (width <= 0) return ATOMA_ERR_SHAPE;
+  hipLaunchKernelGGL(set_rows_kernel, dim3(n_rows), dim3(256), 0, stream, resid, y, bias, width);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int atoma_pack_pair(const float* a, const float* b, void* out, int out_dtype, int n_rows, int width,
+                               hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (width <= 0) return ATOMA_ERR_SHAPE;
+  if (out_dtype == kF32)
+    hipLaunchKernelGGL((pack_pair_kernel<float>), dim3(n_rows), dim3(256), 0, stream, a, b, (float*)out, width);
+  else if (out_dtype == kBF16)
+    hipLaunchKernelGGL((pack_pair_kernel<bf16_t>), dim3(n_rows), dim3(256), 0, stream, a, b, (bf16_t*)out, width);
   else
     return ATOMA_ERR_DTYPE;
   ATOMA_LAUNCH_CHECK();

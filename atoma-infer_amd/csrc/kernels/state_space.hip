@@ -1,0 +1,259 @@
+// A selective state-space recurrence with one scalar decay per head (the Mamba-2 form): per head and request a
+// float32 matrix S [n, vdim] that every token decays, writes and reads,
+//
+//   S <- a S + dt B x^T;   y = S^T C + D x,        a = exp(-exp(A_log) dt),  dt = softplus(dt_raw + dt_bias),
+//
+// with x (vdim per head), B and C (n per group of heads) the token's projections after a short causal convolution over
+// time (with bias) and SiLU.  Everything here is float32.  Four kernels:
+//   ssd_prepare      per token: the convolution (the taps - 1 inputs before an entry's first token come from the
+//                    request's state), bias and SiLU of the x, B, C channels; dt and the decay of every head;
+//   ssd_conv_state   per request: the last taps - 1 inputs of the convolution, for the request's next step;
+//   ssd_scan         per (request, head, 16 columns of S): the recurrence over the entry's tokens in order, S read from
+//                    the request's state slot before and written back after.  A column of S lives in the registers of
+//                    16 neighbouring lanes (n / 16 rows each, rounded up); the tokens' inputs pass LDS in blocks;
+//   ssd_out          per token and norm group: y * silu(z), divided by the root mean square of its group, times the
+//                    weight, in the activation dtype.
+// The order of every sum depends on the sizes alone, so a token's result does not depend on how the request was cut
+// into steps or on what else the step holds.
+//
+// State of a request (float32, one row of the state tensor):  [taps - 1][conv channels]  then  [heads][vdim][n].
+#include "common.h"
+
+using namespace atoma;
+
+struct SsdShape {
+  int heads, groups, vdim, n, taps;
+  int ldp;                          // row stride of the projections
+  int off_z, off_x, off_dt;         // first columns of z, of the convolved channels (x, B, C) and of dt in a row
+};
+
+__device__ __forceinline__ float ssd_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float ssd_softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+// conv channels: x (heads * vdim), then B (groups * n), then C (the same), as they lie in a row of the projections
+__global__ void __launch_bounds__(256)
+ssd_prepare_kernel(const float* __restrict__ proj, SsdShape sh, const int32_t* __restrict__ token_seq,
+                   const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
+                   const float* __restrict__ state, size_t state_stride, const float* __restrict__ taps_w,
+                   const float* __restrict__ conv_bias, const float* __restrict__ dt_bias,
+                   const float* __restrict__ a_log, float* __restrict__ xbc, float* __restrict__ dt,
+                   float* __restrict__ decay) {
+  const int t = blockIdx.x;
+  const int e = token_seq[t];
+  const int i = t - q_start[e];        // the token's index inside its entry
+  const int channels = sh.heads * sh.vdim + 2 * sh.groups * sh.n;
+  if (blockIdx.y == gridDim.y - 1) {
+    // the token's last workgroup: step sizes and decays, which need nothing of the convolution
+    for (int h = threadIdx.x; h < sh.heads; h += 256) {
+      const float d = ssd_softplus(proj[(size_t)t * sh.ldp + sh.off_dt + h] + dt_bias[h]);
+      dt[(size_t)t * sh.heads + h] = d;
+      decay[(size_t)t * sh.heads + h] = expf(-expf(a_log[h]) * d);
+    }
+    return;
+  }
+  const float* conv_state = state + (size_t)state_slots[e] * state_stride;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= channels) return;
+  float y = conv_bias[c];
+  for (int j = 0; j < sh.taps; ++j) {
+    const int s = i - (sh.taps - 1) + j;      // index inside the entry of the input under tap j
+    const float x = s >= 0 ? proj[(size_t)(t - (sh.taps - 1) + j) * sh.ldp + sh.off_x + c]
+                           : conv_state[(size_t)(sh.taps - 1 + s) * channels + c];
+    y = fmaf(taps_w[(size_t)c * sh.taps + j], x, y);
+  }
+  xbc[(size_t)t * channels + c] = y * ssd_sigmoid(y);
+}
+
+// one thread a (entry, channel): the state's rows in ascending order, so that a row is read before it is overwritten
+__global__ void __launch_bounds__(256)
+ssd_conv_state_kernel(const float* __restrict__ proj, SsdShape sh, const int32_t* __restrict__ q_start,
+                      const int32_t* __restrict__ state_slots, float* __restrict__ state, size_t state_stride) {
+  const int e = blockIdx.y;
+  const int channels = sh.heads * sh.vdim + 2 * sh.groups * sh.n;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= channels) return;
+  const int first = q_start[e], count = q_start[e + 1] - first;
+  float* st = state + (size_t)state_slots[e] * state_stride;
+  const int keep = sh.taps - 1;
+  for (int r = 0; r < keep; ++r) {
+    const int s = count - keep + r;     // index inside the entry of the input that row r holds afterwards
+    st[(size_t)r * channels + c] = s >= 0 ? proj[(size_t)(first + s) * sh.ldp + sh.off_x + c]
+                                          : st[(size_t)(r + count) * channels + c];
+  }
+}
+
+constexpr int kScanTokens = 16;      // tokens whose inputs wait in LDS at a time
+constexpr int kScanCols = 16;        // columns of S a workgroup owns
+
+// Sum over 16 neighbouring lanes; every lane gets the same sum (the pairs of each step add the same two numbers).
+__device__ __forceinline__ float lanes16_sum(float x) {
+  x += __shfl_xor(x, 1, 64);
+  x += __shfl_xor(x, 2, 64);
+  x += __shfl_xor(x, 4, 64);
+  x += __shfl_xor(x, 8, 64);
+  return x;
+}
+
+// R: rows of S a lane holds; lane l of a column owns rows l, l + 16, l + 32, ...
+template <int R>
+__global__ void __launch_bounds__(256)
+ssd_scan_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, const float* __restrict__ decay,
+                const float* __restrict__ d_skip, SsdShape sh, const int32_t* __restrict__ q_start,
+                const int32_t* __restrict__ state_slots, float* __restrict__ state, size_t state_stride,
+                float* __restrict__ y) {
+  __shared__ float sb[kScanTokens][16 * R], sc[kScanTokens][16 * R];
+  __shared__ float sx[kScanTokens][kScanCols], sdt[kScanTokens], sa[kScanTokens];
+  const int e = blockIdx.z, h = blockIdx.y, v0 = blockIdx.x * kScanCols;
+  const int first = q_start[e], count = q_start[e + 1] - first;
+  if (count <= 0) return;
+  const int col = threadIdx.x >> 4, l = threadIdx.x & 15;
+  const int v = v0 + col;
+  const bool live = v < sh.vdim;
+  const int inner = sh.heads * sh.vdim, gn = sh.groups * sh.n, channels = inner + 2 * gn;
+  const int g = h / (sh.heads / sh.groups);
+  float* s_ptr = state + (size_t)state_slots[e] * state_stride + (size_t)(sh.taps - 1) * channels +
+                 ((size_t)h * sh.vdim + (live ? v : 0)) * sh.n;
+  float s[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int row = l + 16 * r;
+    s[r] = (live && row < sh.n) ? s_ptr[row] : 0.f;
+  }
+  const float dh = d_skip[h];
+  for (int t0 = 0; t0 < count; t0 += kScanTokens) {
+    const int nt = count - t0 < kScanTokens ? count - t0 : kScanTokens;
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < nt * 16 * R; idx += 256) {
+      const int tt = idx / (16 * R), row = idx % (16 * R);
+      const size_t base = (size_t)(first + t0 + tt) * channels + inner + (size_t)g * sh.n;
+      sb[tt][row] = row < sh.n ? xbc[base + row] : 0.f;
+      sc[tt][row] = row < sh.n ? xbc[base + gn + row] : 0.f;
+    }
+    for (int idx = threadIdx.x; idx < nt * kScanCols; idx += 256) {
+      const int tt = idx / kScanCols, cc = idx % kScanCols;
+      sx[tt][cc] = v0 + cc < sh.vdim ? xbc[(size_t)(first + t0 + tt) * channels + (size_t)h * sh.vdim + v0 + cc] : 0.f;
+    }
+    if (threadIdx.x < nt) {
+      sdt[threadIdx.x] = dt[(size_t)(first + t0 + threadIdx.x) * sh.heads + h];
+      sa[threadIdx.x] = decay[(size_t)(first + t0 + threadIdx.x) * sh.heads + h];
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float a = sa[tt], xv = sx[tt][col], w = sdt[tt] * xv;
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        s[r] = fmaf(a, s[r], w * sb[tt][l + 16 * r]);
+        acc = fmaf(s[r], sc[tt][l + 16 * r], acc);
+      }
+      acc = lanes16_sum(acc);
+      if (l == 0 && live) y[(size_t)(first + t0 + tt) * inner + (size_t)h * sh.vdim + v] = acc + dh * xv;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int row = l + 16 * r;
+      if (row < sh.n) s_ptr[row] = s[r];
+    }
+  }
+}
+
+// one workgroup per (token, norm group)
+template <typename TO>
+__global__ void __launch_bounds__(256)
+ssd_out_kernel(const float* __restrict__ y, const float* __restrict__ proj, int ldp, int off_z,
+               const float* __restrict__ w, float eps, int inner, int part, TO* __restrict__ out) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x, p0 = blockIdx.y * part;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < part; i += 256) {
+    const float z = proj[(size_t)t * ldp + off_z + p0 + i];
+    const float u = y[(size_t)t * inner + p0 + i] * (z * ssd_sigmoid(z));
+    ss = fmaf(u, u, ss);
+  }
+  ss = block_sum<4>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)part + eps);
+  for (int i = threadIdx.x; i < part; i += 256) {
+    const float z = proj[(size_t)t * ldp + off_z + p0 + i];
+    const float u = y[(size_t)t * inner + p0 + i] * (z * ssd_sigmoid(z));
+    out[(size_t)t * inner + p0 + i] = from_f32<TO>(u * inv * w[p0 + i]);
+  }
+}
+
+static bool shape_ok(const SsdShape& sh) {
+  return sh.heads > 0 && sh.groups > 0 && sh.heads % sh.groups == 0 && sh.vdim > 0 && sh.n > 0 && sh.n <= 256 &&
+         sh.taps >= 1 && sh.taps <= 64 && sh.ldp > 0 && sh.off_z >= 0 && sh.off_x >= 0 && sh.off_dt >= 0;
+}
+
+extern "C" int atoma_ssd_prepare(const float* proj, int ldp, int off_z, int off_x, int off_dt, int heads, int groups,
+                                 int vdim, int n, int taps, const int32_t* token_seq, const int32_t* q_start,
+                                 const int32_t* state_slots, const float* state, size_t state_stride,
+                                 const float* taps_w, const float* conv_bias, const float* dt_bias,
+                                 const float* a_log, float* xbc, float* dt, float* decay, int n_tokens,
+                                 hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  SsdShape sh{heads, groups, vdim, n, taps, ldp, off_z, off_x, off_dt};
+  if (!shape_ok(sh)) return ATOMA_ERR_SHAPE;
+  const int channels = heads * vdim + 2 * groups * n;
+  const int blocks = (channels + 255) / 256 + 1;
+  if (blocks > 65535) return ATOMA_ERR_SHAPE;
+  hipLaunchKernelGGL(ssd_prepare_kernel, dim3(n_tokens, blocks), dim3(256), 0, stream, proj, sh, token_seq, q_start,
+                     state_slots, state, state_stride, taps_w, conv_bias, dt_bias, a_log, xbc, dt, decay);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int atoma_ssd_conv_state(const float* proj, int ldp, int off_x, int heads, int groups, int vdim, int n,
+                                    int taps, const int32_t* q_start, const int32_t* state_slots, float* state,
+                                    size_t state_stride, int n_entries, hipStream_t stream) {
+  if (n_entries <= 0 || taps <= 1) return 0;
+  SsdShape sh{heads, groups, vdim, n, taps, ldp, 0, off_x, 0};
+  if (!shape_ok(sh) || n_entries > 65535) return ATOMA_ERR_SHAPE;
+  const int channels = heads * vdim + 2 * groups * n;
+  hipLaunchKernelGGL(ssd_conv_state_kernel, dim3((channels + 255) / 256, n_entries), dim3(256), 0, stream, proj, sh,
+                     q_start, state_slots, state, state_stride);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int atoma_ssd_scan(const float* xbc, const float* dt, const float* decay, const float* d_skip, int heads,
+                              int groups, int vdim, int n, int taps, const int32_t* q_start,
+                              const int32_t* state_slots, float* state, size_t state_stride, float* y,
+                              int n_entries, hipStream_t stream) {
+  if (n_entries <= 0) return 0;
+  SsdShape sh{heads, groups, vdim, n, taps, 1, 0, 0, 0};
+  if (!shape_ok(sh) || n_entries > 65535 || heads > 65535) return ATOMA_ERR_SHAPE;
+  dim3 grid((vdim + kScanCols - 1) / kScanCols, heads, n_entries), block(256);
+  const int rows = (n + 15) / 16;
+#define ATOMA_SCAN(R)                                                                                              \
+  hipLaunchKernelGGL((ssd_scan_kernel<R>), grid, block, 0, stream, xbc, dt, decay, d_skip, sh, q_start, state_slots, \
+                     state, state_stride, y)
+  if (rows <= 1) ATOMA_SCAN(1);
+  else if (rows <= 2) ATOMA_SCAN(2);
+  else if (rows <= 3) ATOMA_SCAN(3);
+  else if (rows <= 4) ATOMA_SCAN(4);
+  else if (rows <= 6) ATOMA_SCAN(6);
+  else if (rows <= 8) ATOMA_SCAN(8);
+  else if (rows <= 12) ATOMA_SCAN(12);
+  else ATOMA_SCAN(16);
+#undef ATOMA_SCAN
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int atoma_ssd_out(const float* y, const float* proj, int ldp, int off_z, const float* w, float eps,
+                             int inner, int norm_groups, void* out, int out_dtype, int n_tokens, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (inner <= 0 || norm_groups <= 0 || inner % norm_groups || norm_groups > 65535 || ldp < inner) return ATOMA_ERR_SHAPE;
+  const int part = inner / norm_groups;
+  dim3 grid(n_tokens, norm_groups), block(256);
+  if (out_dtype == kF32)
+    hipLaunchKernelGGL((ssd_out_kernel<float>), grid, block, 0, stream, y, proj, ldp, off_z, w, eps, inner, part, (float*)out);
+  else if (out_dtype == kBF16)
+    hipLaunchKernelGGL((ssd_out_kernel<bf16_t>), grid, block, 0, stream, y, proj, ldp, off_z, w, eps, inner, part, (bf16_t*)out);
+  else
+    return ATOMA_ERR_DTYPE;
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}

@@ -52,6 +52,8 @@ HIP_MODULES: Dict[str, Tuple[Sequence[str], Sequence[str]]] = {
     "layer_norms": (("norm_sandwich.hip", "qk_norm_rope.hip"), ()),
     "delta_rule": (("delta_rule.hip",), ()),
     "experts": (("experts.hip",), ()),
+    "state_space": (("state_space.hip",), ()),
+    "latent": (("latent.hip",), ()),
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}

@@ -301,18 +301,20 @@ def _term(delta: torch.Tensor, t: int, width: int):
     return _p(delta), _code(delta, "term"), planes, ctypes.c_size_t(t * width)
 
 
-def add_normed(resid: torch.Tensor, terms, w_post: torch.Tensor, eps_post: float,
+def add_normed(resid: torch.Tensor, terms, w_post: Optional[torch.Tensor], eps_post: float,
                w_next: Optional[torch.Tensor] = None, eps_next: float = 0.0,
                out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
     """resid += rmsnorm(sum_i scale_i * term_i) * w_post (float32, in place); with ``w_next`` also returns
     rmsnorm(resid) * w_next in ``out_dtype``.  ``terms``: one or two (tensor, scale) pairs, each tensor [T, W] or
-    planes [S, T, W] (summed), float32 or bfloat16.  Norm weights are float32."""
+    planes [S, T, W] (summed), float32 or bfloat16.  Norm weights are float32.  Without ``w_post`` the sum joins the
+    stream as it is: resid += sum_i scale_i * term_i."""
     _need(resid.dtype is torch.float32 and resid.dim() == 2 and resid.is_contiguous(), "resid must be float32 [T, W]")
     t, width = resid.shape
     _need(1 <= len(terms) <= 2, "one or two terms")
     _need(width <= 16000, "rows of more than 16,000 columns do not fit the kernel's row buffer")
     _dev(resid, w_post, w_next, *[d for d, _ in terms])
-    _f32(w_post, "norm weight", width)
+    if w_post is not None:
+        _f32(w_post, "norm weight", width)
     out = None
     if w_next is not None:
         _f32(w_next, "norm weight", width)
@@ -323,6 +325,29 @@ def add_normed(resid: torch.Tensor, terms, w_post: torch.Tensor, eps_post: float
         _p(resid), *a, ctypes.c_float(terms[0][1]), *b, ctypes.c_float(terms[1][1] if len(terms) > 1 else 0.0),
         _p(w_post), ctypes.c_float(eps_post), _p(w_next), ctypes.c_float(eps_next), _p(out),
         _code(out, "out") if out is not None else F32, t, width, _stream()), "add_normed")
+    return out
+
+
+def set_rows(resid: torch.Tensor, y: torch.Tensor, bias: torch.Tensor) -> None:
+    """resid[t] = y[t] + bias, all float32: the stream's rows replaced by a map of them."""
+    _dev(resid, y, bias)
+    _need(resid.dtype is torch.float32 and resid.dim() == 2 and resid.is_contiguous(), "resid must be float32 [T, W]")
+    t, width = resid.shape
+    _f32(y, "the new rows", t * width)
+    _f32(bias, "the bias row", width)
+    _check(_module("layer_norms").atoma_set_rows(_p(resid), _p(y), _p(bias), t, width, _stream()), "set_rows")
+
+
+def pack_pair(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """[a | b] row by row in ``out_dtype`` for two float32 streams [T, W]."""
+    _dev(a, b)
+    _need(a.dim() == 2 and a.shape == b.shape, "pack_pair: two streams of one shape")
+    _f32(a, "stream")
+    _f32(b, "stream")
+    t, width = a.shape
+    out = torch.empty((t, 2 * width), dtype=out_dtype, device=a.device)
+    _check(_module("layer_norms").atoma_pack_pair(_p(a), _p(b), _p(out), _code(out, "out"), t, width, _stream()),
+           "pack_pair")
     return out
 
 
@@ -454,6 +479,150 @@ def delta_out(o: torch.Tensor, gate_pre: torch.Tensor, w: torch.Tensor, eps: flo
                                                  _p(w), ctypes.c_float(eps), _p(out),
                                                  _code(out, "out"), t, heads, vdim, _stream()), "delta_out")
     return out
+
+
+# ---- a state-space recurrence with a scalar decay per head (state_space.hip) ----------------------------------------
+
+def _ssd_state_ok(state, heads, groups, vdim, n, taps):
+    channels = heads * vdim + 2 * groups * n
+    _need(state.dtype is torch.float32 and state.dim() == 2 and state.is_contiguous()
+          and state.shape[1] == (taps - 1) * channels + heads * vdim * n, "state: bad shape")
+    _need(0 < n <= 256 and 1 <= taps <= 64 and heads % groups == 0, "state sizes up to 256 and up to 64 taps")
+    return channels
+
+
+def ssd_prepare(proj: torch.Tensor, offsets, heads: int, groups: int, vdim: int, n: int, taps: int,
+                token_seq: torch.Tensor, q_start: torch.Tensor, state_slots: torch.Tensor, state: torch.Tensor,
+                taps_w: torch.Tensor, conv_bias: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor):
+    """The inputs of the recurrence for every token: (xbc [T, channels] after convolution, bias and SiLU; dt [T, heads]
+    = softplus(raw + dt_bias); decay [T, heads] = exp(-exp(A_log) dt)), all float32, from ``proj`` float32 [T, ld]
+    whose columns ``offsets`` = (z, first convolved channel, dt) name."""
+    _dev(proj, token_seq, q_start, state_slots, state, taps_w, conv_bias, dt_bias, a_log)
+    t, s = proj.shape[0], state_slots.numel()
+    channels = _ssd_state_ok(state, heads, groups, vdim, n, taps)
+    off_z, off_x, off_dt = (int(o) for o in offsets)
+    _need(proj.dtype is torch.float32 and proj.dim() == 2 and proj.stride(1) == 1, "proj must be float32 [T, ld]")
+    _need(min(off_z, off_x, off_dt) >= 0 and max(off_z + heads * vdim, off_x + channels, off_dt + heads) <= proj.shape[1],
+          "the projections' columns do not fit proj")
+    _i32(token_seq, "token_seq", t)
+    _i32(q_start, "q_start", s + 1)
+    _i32(state_slots, "state_slots", s)
+    _f32(taps_w, "taps", channels * taps)
+    _f32(conv_bias, "the convolution's bias", channels)
+    _f32(dt_bias, "dt_bias", heads)
+    _f32(a_log, "A_log", heads)
+    dev = proj.device
+    xbc = torch.empty((t, channels), dtype=torch.float32, device=dev)
+    dt = torch.empty((t, heads), dtype=torch.float32, device=dev)
+    decay = torch.empty((t, heads), dtype=torch.float32, device=dev)
+    _check(_module("state_space").atoma_ssd_prepare(
+        _p(proj), proj.stride(0), off_z, off_x, off_dt, heads, groups, vdim, n, taps, _p(token_seq), _p(q_start),
+        _p(state_slots), _p(state), ctypes.c_size_t(state.stride(0)), _p(taps_w), _p(conv_bias), _p(dt_bias), _p(a_log),
+        _p(xbc), _p(dt), _p(decay), t, _stream()), "ssd_prepare")
+    return xbc, dt, decay
+
+
+def ssd_conv_state(proj: torch.Tensor, off_x: int, heads: int, groups: int, vdim: int, n: int, taps: int,
+                   q_start: torch.Tensor, state_slots: torch.Tensor, state: torch.Tensor) -> None:
+    """The last ``taps - 1`` inputs of the convolution of every entry into its request's state row (an entry shorter
+    than that shifts the old rows)."""
+    _dev(proj, q_start, state_slots, state)
+    s = state_slots.numel()
+    channels = _ssd_state_ok(state, heads, groups, vdim, n, taps)
+    _need(proj.dtype is torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and 0 <= off_x
+          and off_x + channels <= proj.shape[1], "proj must be float32 [T, ld] and hold the channels")
+    _i32(q_start, "q_start", s + 1)
+    _i32(state_slots, "state_slots", s)
+    _check(_module("state_space").atoma_ssd_conv_state(
+        _p(proj), proj.stride(0), int(off_x), heads, groups, vdim, n, taps, _p(q_start), _p(state_slots), _p(state),
+        ctypes.c_size_t(state.stride(0)), s, _stream()), "ssd_conv_state")
+
+
+def ssd_scan(xbc: torch.Tensor, dt: torch.Tensor, decay: torch.Tensor, d_skip: torch.Tensor, heads: int, groups: int,
+             vdim: int, n: int, taps: int, q_start: torch.Tensor, state_slots: torch.Tensor,
+             state: torch.Tensor) -> torch.Tensor:
+    """The recurrence over every entry's tokens, from and into the requests' state rows; returns y float32
+    [T, heads vdim] = S^T C + D x."""
+    _dev(xbc, dt, decay, d_skip, q_start, state_slots, state)
+    t, s = xbc.shape[0], state_slots.numel()
+    channels = _ssd_state_ok(state, heads, groups, vdim, n, taps)
+    _need(xbc.dtype is torch.float32 and xbc.is_contiguous() and tuple(xbc.shape) == (t, channels), "xbc: bad shape")
+    for x, what in ((dt, "dt"), (decay, "decay")):
+        _need(x.dtype is torch.float32 and x.is_contiguous() and tuple(x.shape) == (t, heads), f"{what}: bad shape")
+    _f32(d_skip, "D", heads)
+    _i32(q_start, "q_start", s + 1)
+    _i32(state_slots, "state_slots", s)
+    y = torch.empty((t, heads * vdim), dtype=torch.float32, device=xbc.device)
+    _check(_module("state_space").atoma_ssd_scan(
+        _p(xbc), _p(dt), _p(decay), _p(d_skip), heads, groups, vdim, n, taps, _p(q_start), _p(state_slots), _p(state),
+        ctypes.c_size_t(state.stride(0)), _p(y), s, _stream()), "ssd_scan")
+    return y
+
+
+def ssd_out(y: torch.Tensor, proj: torch.Tensor, off_z: int, w: torch.Tensor, eps: float, norm_groups: int,
+            out_dtype: torch.dtype) -> torch.Tensor:
+    """u = y * silu(z) with z the columns of ``proj`` from ``off_z`` on; u divided by the root mean square of each of
+    its ``norm_groups`` equal parts, times w, in ``out_dtype``."""
+    _dev(y, proj, w)
+    t, inner = y.shape
+    _need(y.dtype is torch.float32 and y.is_contiguous(), "y: bad shape")
+    _need(proj.dtype is torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[0] == t
+          and 0 <= off_z and off_z + inner <= proj.shape[1], "proj must be float32 [T, ld] and hold z")
+    _need(norm_groups > 0 and inner % norm_groups == 0, "the norm's groups must divide the row")
+    _f32(w, "norm weight", inner)
+    out = torch.empty((t, inner), dtype=out_dtype, device=y.device)
+    _check(_module("state_space").atoma_ssd_out(_p(y), _p(proj), proj.stride(0), int(off_z), _p(w), ctypes.c_float(eps),
+                                                inner, int(norm_groups), _p(out), _code(out, "out"), t, _stream()),
+           "ssd_out")
+    return out
+
+
+# ---- attention over one cached latent vector per token (latent.hip) ---------------------------------------------------
+
+def latent_prepare(proj: torch.Tensor, offsets, heads: int, dim: int, rank: int, rank_p: int, w_norm: torch.Tensor,
+                   eps: float, kcache: torch.Tensor, vcache: torch.Tensor, slot_mapping: torch.Tensor, page_size: int,
+                   act_dtype: torch.dtype):
+    """(q [T, heads dim] in ``act_dtype``, gate float32 [T, heads] = sigmoid) from ``proj`` float32 [T, ld] whose
+    columns ``offsets`` = (q, down projection, gates) name; the normed down projection (rank numbers, zeros up to
+    ``rank_p``) goes into both tiles of the token's cache slot."""
+    _dev(proj, w_norm, kcache, vcache, slot_mapping)
+    t = proj.shape[0]
+    off_q, off_c, off_g = (int(o) for o in offsets)
+    _need(proj.dtype is torch.float32 and proj.dim() == 2 and proj.stride(1) == 1, "proj must be float32 [T, ld]")
+    _need(min(off_q, off_c, off_g) >= 0 and max(off_q + heads * dim, off_c + rank, off_g + heads) <= proj.shape[1],
+          "the projections' columns do not fit proj")
+    _f32(w_norm, "norm weight", rank)
+    _i32(slot_mapping, "slot_mapping", t)
+    pages = kcache.shape[0]
+    _need(kcache.is_contiguous() and vcache.is_contiguous() and tuple(kcache.shape) == (pages, 1, page_size * rank_p)
+          and tuple(vcache.shape) == (pages, 1, page_size * rank_p) and kcache.dtype is vcache.dtype
+          and kcache.dtype is act_dtype, "cache tensors must be [pages, 1, page_size * rank] tiles of the activation dtype")
+    q = torch.empty((t, heads * dim), dtype=act_dtype, device=proj.device)
+    gate = torch.empty((t, heads), dtype=torch.float32, device=proj.device)
+    _check(_module("latent").atoma_latent_prepare(
+        _p(proj), proj.stride(0), off_q, off_c, off_g, heads * dim, rank, rank_p, heads, _p(w_norm), ctypes.c_float(eps),
+        _p(kcache), _p(vcache), _code(kcache, "cache"), _p(slot_mapping), page_size, _p(q), _code(q, "q"), _p(gate), t,
+        _stream()), "latent_prepare")
+    return q, gate
+
+
+def head_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gate: Optional[torch.Tensor] = None,
+                ) -> torch.Tensor:
+    """Per head a product of its own: x [T, H K] (row stride free), w [H, N, K] -> [T, H N] in ``out_dtype``, float32
+    sums; with ``gate`` float32 [T, H] every head's result is multiplied by its number."""
+    _dev(x, w, gate)
+    _need(w.dim() == 3 and w.is_contiguous(), "head_linear: w must be contiguous [H, N, K]")
+    h, n, k = w.shape
+    t = x.shape[0]
+    _need(x.dim() == 2 and x.stride(1) == 1 and x.shape[1] == h * k, "head_linear: x must be [T, H K]")
+    if gate is not None:
+        _f32(gate, "gate", t * h)
+    out = torch.empty((t, h * n), dtype=out_dtype, device=x.device)
+    _check(_module("latent").atoma_head_linear(_p(x), _code(x, "x"), x.stride(0) if t > 1 else h * k, _p(w), _code(w, "w"),
+                                               _p(out), _code(out, "out"), h * n, _p(gate), t, h, k, n, _stream()),
+           "head_linear")
+    return out
+
 
 
 def route_topk(logits: torch.Tensor, top: int):

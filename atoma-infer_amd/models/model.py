@@ -28,6 +28,8 @@ class Model:
     spec: ModelSpec
     device: torch.device
     act_dtype: torch.dtype
+    #: for whoever looks into a step: called as ``after_block(run-order position, stream, what is still pending)``
+    after_block: Optional[object] = None
 
     @property
     def vocab_size(self) -> int:
@@ -47,11 +49,24 @@ class Model:
         first = blocks[0].entry_norm() if blocks else None
         resid, pending = spec.embedding[1].forward(ctx.tokens, first) if first is not None else \
             (spec.embedding[1].forward(ctx.tokens), None)
+        # a block that maps the stream from the embedding's rows too gets them as they were (gathered once more: the
+        # stream's own rows are summed into in place), and one that is run several times is told which run this is
+        embedded = spec.embedding[1].forward(ctx.tokens) if any(getattr(b, "reads_embedding", False) for b in blocks) \
+            else None
+        runs = {}
         for pos, block in enumerate(blocks):
+            extra = {}
             if block.fuses_next_norm:
-                pending = block.forward(resid, pending, ctx, ctx.layer_cache(pos), next_norm=readers[pos])
-            else:
-                pending = block.forward(resid, pending, ctx, ctx.layer_cache(pos))
+                extra["next_norm"] = readers[pos]
+            if getattr(block, "reads_embedding", False):
+                extra["embedded"] = embedded
+            if getattr(block, "takes_turn", False):
+                layer = spec.run_order[pos].layer
+                extra["turn"] = runs.get(layer, 0)
+                runs[layer] = extra["turn"] + 1
+            pending = block.forward(resid, pending, ctx, ctx.layer_cache(pos), **extra)
+            if self.after_block is not None:
+                self.after_block(pos, resid, pending)
         if ctx.n_want == 0:
             return None
         if isinstance(pending, Begun):      # the final norm, begun by the last product, on every row

@@ -2,8 +2,9 @@
 from .base import (Block, CacheSpec, FeedForward, Mixer, Norm, Part, PositionEncoding, StateSpec, WeightSpec,
                    make_part, register_block, register_feed_forward, register_mixer, register_norm,
                    register_position, registered_kinds)
-from .attention import PagedAttention, TiedValueAttention
-from .block import PreNormBlock, SandwichBlock
+from .attention import LatentAttention, PagedAttention, TiedValueAttention
+from .block import PreNormBlock, SandwichBlock, SideBySideBlock
+from .loop import LoopEntry, NoMixer
 from .embedding import OutputHead, TokenEmbedding
 from .experts import RoutedExperts
 from .feed_forward import SwiGLU
@@ -11,10 +12,11 @@ from .linear import linear
 from .norm import RMSNorm
 from .parallel import ParallelMixer
 from .position import NoPosition, RotaryEncoding
-from .recurrent import GatedDeltaRule
+from .recurrent import GatedDeltaRule, StateSpaceDuality
 
 __all__ = ["Block", "CacheSpec", "FeedForward", "Mixer", "Norm", "Part", "PositionEncoding", "StateSpec",
            "WeightSpec", "make_part", "register_block", "register_feed_forward", "register_mixer", "register_norm",
            "register_position", "registered_kinds", "PagedAttention", "PreNormBlock", "OutputHead",
            "TokenEmbedding", "SwiGLU", "linear", "RMSNorm", "NoPosition", "RotaryEncoding", "TiedValueAttention",
-           "SandwichBlock", "RoutedExperts", "ParallelMixer", "GatedDeltaRule"]
+           "SandwichBlock", "RoutedExperts", "ParallelMixer", "GatedDeltaRule", "LatentAttention", "SideBySideBlock",
+           "LoopEntry", "NoMixer", "StateSpaceDuality"]

@@ -29,9 +29,17 @@ from .linear import as_tensor, linear, linear_delta
 class PagedAttention(Mixer):
     def __init__(self, width: int, num_heads: int, num_kv_heads: int, head_size: int,
                  position: Optional[PositionEncoding] = None, window: Optional[int] = None,
-                 scale: Optional[float] = None, chunk: Optional[int] = None):
+                 scale: Optional[float] = None, chunk: Optional[int] = None, value_size: Optional[int] = None,
+                 names=("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight")):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads cannot be grouped over {num_kv_heads} KV heads")
+        # ``value_size``: columns of a value head where they differ from a key head's; ``names``: the tensors of the
+        # four projections below the part's prefix.  The kernels and the cache see one head size: where keys and values
+        # differ, or the size is no multiple of 8, both run as the next multiple of 16 of the larger (``self.hd``;
+        # zero rows in the projections, zero columns in the output projection, which changes no score and no output)
+        self.hd_in, self.vd_in, self.names = int(head_size), int(value_size or head_size), tuple(names)
+        if self.vd_in != self.hd_in or self.hd_in % 8:
+            head_size = -(-max(self.hd_in, self.vd_in) // 16) * 16
         # every multiple of 8 up to 256, as the reference's kernels take (csrc/src/lib.rs:136-143, 790)
         if head_size % 8 or not 8 <= head_size <= 256:
             raise ValueError(f"head size {head_size} is not supported: the attention kernels take multiples of 8 "
@@ -46,7 +54,7 @@ class PagedAttention(Mixer):
         # chunk c: the token at p sees keys (p // c) * c .. p only, chunks counted from the request's first position
         self.chunk = chunk
         self.sinks: Optional[torch.Tensor] = None       # float32 [heads]: exp(sinks[h]) joins the softmax denominator
-        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd_in)
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
         self.w_qkv_tiled = self.w_o_tiled = None
@@ -60,15 +68,26 @@ class PagedAttention(Mixer):
         return self.position is None or self.position.graph_safe()
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        q, kv = self.nh * self.hd, self.nkv * self.hd
-        return {"q_proj.weight": WeightSpec((q, self.width)), "k_proj.weight": WeightSpec((kv, self.width)),
-                "v_proj.weight": WeightSpec((kv, self.width)), "o_proj.weight": WeightSpec((self.width, q))}
+        n = self.names
+        return {n[0]: WeightSpec((self.nh * self.hd_in, self.width)), n[1]: WeightSpec((self.nkv * self.hd_in, self.width)),
+                n[2]: WeightSpec((self.nkv * self.vd_in, self.width)), n[3]: WeightSpec((self.width, self.nh * self.vd_in))}
+
+    @staticmethod
+    def _pad_heads(w: torch.Tensor, heads: int, size: int, to: int, rows: bool) -> torch.Tensor:
+        """``w`` with every head's ``size`` rows (or columns) followed by zeros up to ``to``."""
+        if size == to:
+            return w
+        if rows:
+            return torch.nn.functional.pad(w.view(heads, size, w.shape[1]), (0, 0, 0, to - size)).reshape(heads * to, -1)
+        return torch.nn.functional.pad(w.view(w.shape[0], heads, size), (0, to - size)).reshape(w.shape[0], heads * to)
 
     def cache_spec(self) -> CacheSpec:
         return CacheSpec(self.nkv, self.hd, self.window, chunk=self.chunk)
 
     def load(self, get, device, act_dtype) -> None:
-        ws = [get("q_proj.weight"), get("k_proj.weight"), get("v_proj.weight")]
+        ws = [self._pad_heads(get(self.names[0]), self.nh, self.hd_in, self.hd, True),
+              self._pad_heads(get(self.names[1]), self.nkv, self.hd_in, self.hd, True),
+              self._pad_heads(get(self.names[2]), self.nkv, self.vd_in, self.hd, True)]
         dt = ws[0].dtype if all(w.dtype is ws[0].dtype for w in ws) else torch.float32
         if self.position is not None:
             self.position.load(get, device, act_dtype)
@@ -85,7 +104,7 @@ class PagedAttention(Mixer):
             ws[0] = ws[0].reshape(self.nh, self.hd, self.width)[:, order].reshape(self.nh * self.hd, self.width)
             ws[1] = ws[1].reshape(self.nkv, self.hd, self.width)[:, order].reshape(self.nkv * self.hd, self.width)
         self.w_qkv = torch.cat([w.to(device=device, dtype=dt) for w in ws], dim=0).contiguous()
-        self.w_o = get("o_proj.weight").to(device).contiguous()
+        self.w_o = self._pad_heads(get(self.names[3]), self.nh, self.vd_in, self.hd, False).to(device).contiguous()
         self.act_dtype = act_dtype
         # second copies in the order in which the kernels of steps of few rows read them
         self.w_qkv_tiled = self.w_o_tiled = None
@@ -209,9 +228,9 @@ class TiedValueAttention(PagedAttention):
     def __init__(self, width: int, num_heads: int, num_kv_heads: int, head_size: int, scale: float, norm_eps: float,
                  rotary_base: float, rotary_dim: int, chunk: Optional[int] = None, window: Optional[int] = None,
                  sink: bool = True):
-        self.hd_in = int(head_size)
-        padded = -(-self.hd_in // 16) * 16      # (multiples of 16: what the matrix-core kernel takes)
+        padded = -(-int(head_size) // 16) * 16      # (multiples of 16: what the matrix-core kernel takes)
         super().__init__(width, num_heads, num_kv_heads, padded, None, window, scale, chunk)
+        self.hd_in = self.vd_in = int(head_size)
         if head_size % 2 or rotary_dim % 2 or not 0 <= rotary_dim <= head_size or rotary_dim > 256:
             raise ValueError(f"rotary_dim {rotary_dim} must be even, at most the head size {head_size} and at most 256")
         self.norm_eps, self.rotary_base, self.rotary_dim, self.has_sink = float(norm_eps), float(rotary_base), \
@@ -274,5 +293,92 @@ class TiedValueAttention(PagedAttention):
         return linear_delta(out, self.w_o, None, self.w_o_tiled)
 
 
+class LatentAttention(PagedAttention):
+    """Attention whose keys and values of every head are products of one small vector per token, the only thing the
+    cache keeps:
+
+    * q = W_q x (``heads`` heads of ``head_size``); c = norm(W_dkv x), ``rank`` numbers, RMS-normed with the plain
+      weight ``dkv.norm``; per head k = W_uk c and v = W_uv c (``value_size`` columns);
+    * no positions are encoded; a token sees every key up to its own; one learned sink per head joins the softmax
+      denominator (tensor ``sink``);
+    * a head's output is multiplied by sigmoid(W_g x)_head; then W_o.
+
+    The heads' key and value maps are moved to the query's side, ``(W_uk c) . q = c . (W_uk^T q)`` and
+    ``sum_j p_j W_uv c_j = W_uv sum_j p_j c_j``: the framework's attention kernels then run with one shared key/value
+    head of ``rank`` columns (rounded up to a multiple of 16) whose values are its keys, and a decoded token reads
+    ``rank`` numbers per cached token whatever the number of heads.  (The cache keeps c twice, once in the order the
+    kernels read keys and once in that of values.)
+
+    Tensors ([out, in]): ``q``, ``dkv``, ``dkv.norm``, ``uk`` [heads * head_size, rank], ``uv`` [heads * value_size,
+    rank], ``sink`` [heads], ``g`` [heads, width], ``o`` [width, heads * value_size].
+    """
+
+    def __init__(self, width: int, num_heads: int, head_size: int, value_size: int, rank: int, scale: float,
+                 norm_eps: float):
+        rank_p = -(-int(rank) // 16) * 16
+        super().__init__(width, num_heads, 1, rank_p, None, None, scale, None)
+        self.qd, self.vd, self.rank, self.norm_eps = int(head_size), int(value_size), int(rank), float(norm_eps)
+        self.hd_in = self.vd_in = self.rank
+        self.w_in = self.w_uk = self.w_uv = self.c_norm = None
+        self.off_c = self.nh * self.qd
+        self.off_g = self.off_c + self.rank
+
+    def graph_safe(self) -> bool:
+        return True
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        h, w, r = self.nh, self.width, self.rank
+        return {"q": WeightSpec((h * self.qd, w)), "dkv": WeightSpec((r, w)), "dkv.norm": WeightSpec((r,), "norm"),
+                "uk": WeightSpec((h * self.qd, r), std=r ** -0.5), "uv": WeightSpec((h * self.vd, r), std=r ** -0.5),
+                "sink": WeightSpec((h,), "linear", std=1.0), "g": WeightSpec((h, w), std=0.1),
+                "o": WeightSpec((w, h * self.vd))}
+
+    def load(self, get, device, act_dtype) -> None:
+        ws = [get("q"), get("dkv"), get("g")]
+        dt = ws[0].dtype if all(w.dtype is ws[0].dtype for w in ws) else torch.float32
+        rows = sum(w.shape[0] for w in ws)
+        parts = [w.to(device=device, dtype=dt) for w in ws]
+        if (-rows) % 64:      # whole tiles for the matrix-core products
+            parts.append(torch.zeros(((-rows) % 64, self.width), dtype=dt, device=device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        # per head [out, in]: the key map transposed (it acts on the query), padded to the cache's columns with
+        # zero rows; the value map with zero columns under the padding
+        uk = get("uk").to(device).view(self.nh, self.qd, self.rank).transpose(1, 2)
+        self.w_uk = torch.nn.functional.pad(uk, (0, 0, 0, self.hd - self.rank)).contiguous()
+        uv = get("uv").to(device).view(self.nh, self.vd, self.rank)
+        self.w_uv = torch.nn.functional.pad(uv, (0, self.hd - self.rank)).contiguous()
+        f32 = dict(device=device, dtype=torch.float32)
+        self.c_norm = get("dkv.norm").to(**f32).contiguous()
+        self.sinks = get("sink").to(**f32).contiguous()
+        self.w_o = get("o").to(device).contiguous()
+        self.act_dtype = act_dtype
+        self.w_o_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_o.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            self.w_o_tiled = gemm_bf16.tile_copies_resid(self.w_o)
+
+    def device_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_uk, self.w_uv, self.w_o))
+
+    accepts_begun = False
+    takes_sink = False
+
+    def forward(self, x, ctx, cache, sink=None):
+        if not cache.writable:
+            raise NotImplementedError("latent attention reads only a cache of its own")
+        t = x.shape[0]
+        # q, the down projection and the gates leave their product in float32: the norm and the gates are float32 work
+        proj = linear(x, self.w_in, torch.float32)
+        q, gate = ops.latent_prepare(proj, (0, self.off_c, self.off_g), self.nh, self.qd, self.rank, self.hd,
+                                     self.c_norm, self.norm_eps, cache.k, cache.v, cache.slot_mapping,
+                                     cache.page_size, x.dtype)
+        ql = ops.head_linear(q, self.w_uk, x.dtype)                      # the queries in the latent's columns
+        mixed = torch.empty((t, self.nh * self.hd), dtype=x.dtype, device=x.device)
+        self.attend(ql, cache.k, cache.v, mixed, ctx, cache)
+        out = ops.head_linear(mixed, self.w_uv, x.dtype, gate)           # the heads' values, gated
+        return linear_delta(out, self.w_o, None, self.w_o_tiled)
+
+
+register_mixer("latent_attention", LatentAttention)
 register_mixer("attention", PagedAttention)
 register_mixer("tied_value_attention", TiedValueAttention)

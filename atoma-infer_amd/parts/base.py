@@ -235,6 +235,10 @@ class Block(Part):
     #: True if ``forward`` has a keyword ``next_norm``: the norm that will read this block's output (the next
     #: block's ``entry_norm()``, or the final norm), so that the block's last product may begin it
     fuses_next_norm = False
+    #: True if ``forward`` has a keyword ``embedded``: the float32 rows as the embedding left them
+    reads_embedding = False
+    #: True if ``forward`` has a keyword ``turn``: how many calls of this block the run order has before this one
+    takes_turn = False
 
     def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], ctx, cache) -> torch.Tensor:
         """Consume the pending ``delta`` into ``resid`` (float32 [T, width], in place) and return the new pending delta."""

@@ -4,6 +4,9 @@
 stream is float32; each sum is fused with the norm that follows it, so a block receives the previous block's
 output as a pending ``delta`` and returns its own.
 
+``SideBySideBlock``: one norm whose output both sublayers read, ``h = norm1(x)``, ``y = x + (mixer(h) + ffn(h))``; the
+two outputs travel on unsummed, and the kernel of the norm that reads the stream next adds them in.
+
 ``SandwichBlock``: a norm before and a norm behind each sublayer, ``h = x + norm1b(mixer(norm1(x)))``,
 ``y = h + norm2b(ffn(norm2(h)))``; the feed-forward half may be absent.  One kernel norms a sublayer's output, adds
 it to the stream and applies the norm that reads the stream next.
@@ -129,5 +132,40 @@ class SandwichBlock(Block):
         return Normed(x, next_norm) if next_norm is not None else None
 
 
+class SideBySideBlock(Block):
+    """``x += mixer(norm1(x)) + feed_forward(norm1(x))``: one norm, read by both sublayers; the feed-forward may be
+    absent.  ``names``: the children's prefixes below the layer's, in the order (norm, mixer, feed-forward)."""
+
+    def __init__(self, norm1: Norm, mixer: Mixer, feed_forward: Optional[FeedForward] = None,
+                 names=("", "mix", "mlp")):
+        self.norm1, self.mixer, self.feed_forward = norm1, mixer, feed_forward
+        self.names = tuple(names)
+
+    def _children(self):
+        return [(n, p) for n, p in zip(self.names, (self.norm1, self.mixer, self.feed_forward)) if p is not None]
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {_join(n, k): ws for n, part in self._children() for k, ws in part.weight_specs().items()}
+
+    def load(self, get, device, act_dtype) -> None:
+        for n, part in self._children():
+            part.load(lambda rel, _n=n: get(_join(_n, rel)), device, act_dtype)
+
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe() for _, part in self._children())
+
+    def device_bytes(self) -> int:
+        return sum(part.device_bytes() for _, part in self._children())
+
+    def forward(self, resid, delta, ctx, cache):
+        from .base import WeightedSum
+        x = self.norm1.add_norm(resid, delta)
+        a = self.mixer.forward(x, ctx, cache)
+        if self.feed_forward is None:
+            return a
+        return WeightedSum([(a, 1.0), (self.feed_forward.forward(x, ctx), 1.0)])
+
+
 register_block("pre_norm", PreNormBlock)
+register_block("side_by_side", SideBySideBlock)
 register_block("sandwich", SandwichBlock)

@@ -17,8 +17,10 @@ from .linear import linear, linear_delta
 
 
 class SwiGLU(FeedForward):
-    def __init__(self, width: int, intermediate: int):
-        self.width, self.inter = int(width), int(intermediate)
+    def __init__(self, width: int, intermediate: int,
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+        # ``names``: the tensors of the gate, up and down matrices below the part's prefix
+        self.width, self.inter, self.names = int(width), int(intermediate), tuple(names)
         self.block = 0
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_gate_up_tiled = self.w_down_tiled = None
@@ -28,12 +30,12 @@ class SwiGLU(FeedForward):
         return True
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {"gate_proj.weight": WeightSpec((self.inter, self.width)),
-                "up_proj.weight": WeightSpec((self.inter, self.width)),
-                "down_proj.weight": WeightSpec((self.width, self.inter))}
+        return {self.names[0]: WeightSpec((self.inter, self.width)),
+                self.names[1]: WeightSpec((self.inter, self.width)),
+                self.names[2]: WeightSpec((self.width, self.inter))}
 
     def load(self, get, device, act_dtype) -> None:
-        g, u = get("gate_proj.weight"), get("up_proj.weight")
+        g, u = get(self.names[0]), get(self.names[1])
         dt = g.dtype if g.dtype is u.dtype else torch.float32
         g, u = g.to(device=device, dtype=dt), u.to(device=device, dtype=dt)
         self.block = 16 if self.inter % 16 == 0 else 0
@@ -42,7 +44,7 @@ class SwiGLU(FeedForward):
             self.w_gate_up = gu.reshape(2 * self.inter, self.width).contiguous()
         else:
             self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
-        self.w_down = get("down_proj.weight").to(device).contiguous()
+        self.w_down = get(self.names[2]).to(device).contiguous()
         # second copies of the matrices in the order the streaming kernels' waves read them, for steps of few rows
         self.w_gate_up_tiled = self.w_down_tiled = None
         if act_dtype is torch.bfloat16 and self.w_gate_up.dtype is torch.bfloat16 and self.w_down.dtype is torch.bfloat16:

@@ -14,9 +14,11 @@ from .base import Begun, Norm, WeightedSum, WeightSpec, register_norm
 
 
 class RMSNorm(Norm):
-    def __init__(self, width: int, eps: float, name: str = "weight"):
+    def __init__(self, width: int, eps: float, name: str = "weight", offset: float = 0.0):
         # ``name``: the tensor's name below the part's prefix ("weight" as checkpoints of the Llama family have it)
-        self.width, self.eps, self.name = int(width), float(eps), str(name)
+        # ``offset``: what is added to the stored tensor to make the weight (1 for weights stored around zero); such
+        # a weight is kept in float32, since 1 + w has more digits than the checkpoint's dtype
+        self.width, self.eps, self.name, self.offset = int(width), float(eps), str(name), float(offset)
         self.weight: Optional[torch.Tensor] = None
         self.weight_f32: Optional[torch.Tensor] = None
         self.act_dtype = torch.float32
@@ -25,10 +27,12 @@ class RMSNorm(Norm):
         return True
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {self.name: WeightSpec((self.width,), "norm")}
+        return {self.name: WeightSpec((self.width,), "norm" if self.offset == 0.0 else "norm_zero")}
 
     def load(self, get, device, act_dtype) -> None:
         self.weight = get(self.name).to(device).contiguous()
+        if self.offset != 0.0:
+            self.weight = (self.weight.to(torch.float32) + self.offset).contiguous()
         self.weight_f32 = self.weight.to(torch.float32)
         self.act_dtype = act_dtype
 
@@ -36,6 +40,13 @@ class RMSNorm(Norm):
         return self.weight.numel() * self.weight.element_size()
 
     def add_norm(self, resid, delta, rows=None):
+        if isinstance(delta, WeightedSum):
+            # sublayers that ran side by side: their outputs are summed into the stream by the norm's own kernel
+            if rows is None:
+                return ops.add_normed(resid, delta.terms, None, 0.0, self.weight_f32, self.eps, self.act_dtype)
+            # (rows are asked for behind the last block only: the stream takes the sum, then the rows are normed)
+            ops.add_normed(resid, delta.terms, None, 0.0)
+            delta = None
         return ops.add_rmsnorm(resid, delta, self.weight, self.eps, self.act_dtype, rows)
 
     def add_normed(self, resid, delta, next_norm=None):
@@ -51,7 +62,7 @@ class RMSNorm(Norm):
     # the norm begun by its neighbours (bfloat16 steps of at most 16 rows): see kernels/gemm_bf16.py; with many rows
     # the library adds its product to the residual rows itself, and the norm reads them once
     def add_product(self, resid, x, w, tiled=None):
-        if self.act_dtype is not torch.bfloat16 or w.dtype is not torch.bfloat16:
+        if self.act_dtype is not torch.bfloat16 or w.dtype is not torch.bfloat16 or self.weight.dtype is not torch.bfloat16:
             return None
         from ..kernels import gemm_bf16
         from .linear import Normed, as_tensor
@@ -64,7 +75,8 @@ class RMSNorm(Norm):
         return None
 
     def embed(self, table, tokens):
-        if self.act_dtype is not torch.bfloat16 or tokens.numel() > 16 or table.shape[1] != self.width:
+        if self.act_dtype is not torch.bfloat16 or tokens.numel() > 16 or table.shape[1] != self.width \
+                or self.weight.dtype is not torch.bfloat16:
             return None
         resid, u, ss = ops.embed_begin_norm(tokens, table, self.weight)
         return resid, Begun(u, ss, self.eps, self.width, self)

@@ -19,9 +19,15 @@ from .base import PositionEncoding, register_position
 _TABLES: Dict[tuple, Tuple[torch.Tensor, torch.Tensor]] = {}
 
 
-def rotary_inv_freq(head_size: int, theta: float, scaling: Optional[dict]) -> torch.Tensor:
-    """float32 inverse frequencies [head_size / 2]; ``scaling`` holds the llama3 constants or is None."""
-    f32 = torch.float32
+def rotary_inv_freq(head_size: int, theta: float, scaling: Optional[dict], precise: bool = False) -> torch.Tensor:
+    """float32 inverse frequencies [head_size / 2]; ``scaling`` holds the llama3 constants or is None.  ``precise``:
+    worked out in float64 and rounded once, where the default follows the reference's float32 steps."""
+    if precise:
+        return _inv_freq(head_size, theta, scaling, torch.float64).to(torch.float32)
+    return _inv_freq(head_size, theta, scaling, torch.float32)
+
+
+def _inv_freq(head_size: int, theta: float, scaling: Optional[dict], f32: torch.dtype) -> torch.Tensor:
     exps = torch.arange(0, head_size, 2, dtype=f32) / torch.tensor(float(head_size), dtype=f32)
     freq = 1.0 / torch.pow(torch.tensor(float(theta), dtype=f32), exps)
     if scaling is None:
@@ -38,7 +44,8 @@ def rotary_inv_freq(head_size: int, theta: float, scaling: Optional[dict]) -> to
 
 class RotaryEncoding(PositionEncoding):
     def __init__(self, head_size: int, theta: float, max_positions: int, scaling: Optional[dict] = None,
-                 rotary_dim: Optional[int] = None):
+                 rotary_dim: Optional[int] = None, precise: bool = False):
+        self.precise = bool(precise)
         self.head_size, self.theta, self.max_positions = int(head_size), float(theta), int(max_positions)
         self.scaling = dict(scaling) if scaling else None
         self.rotary_dim = int(rotary_dim) if rotary_dim is not None else self.head_size
@@ -48,7 +55,7 @@ class RotaryEncoding(PositionEncoding):
 
     def _key(self, device):
         sc = tuple(sorted(self.scaling.items())) if self.scaling else None
-        return (self.rotary_dim, self.theta, self.max_positions, sc, str(device))
+        return (self.rotary_dim, self.theta, self.max_positions, sc, str(device), self.precise)
 
     def graph_safe(self) -> bool:
         return True
@@ -56,7 +63,7 @@ class RotaryEncoding(PositionEncoding):
     def prepare(self, device) -> None:
         key = self._key(device)
         if key not in _TABLES:
-            inv = rotary_inv_freq(self.rotary_dim, self.theta, self.scaling)
+            inv = rotary_inv_freq(self.rotary_dim, self.theta, self.scaling, self.precise)
             ang = torch.arange(self.max_positions, dtype=torch.float32)[:, None] * inv[None, :]
             _TABLES[key] = (torch.cos(ang).to(device).contiguous(), torch.sin(ang).to(device).contiguous())
         self.cos, self.sin = _TABLES[key]

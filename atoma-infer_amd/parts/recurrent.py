@@ -127,4 +127,88 @@ class GatedDeltaRule(Mixer):
         return linear_delta(y, self.w_o, None, self.w_o_tiled)
 
 
+class StateSpaceDuality(Mixer):
+    """A selective state-space recurrence with one scalar decay per head (the Mamba-2 form): per head a float32 matrix
+    S [state, vdim],
+
+        S <- exp(-exp(A_log) dt) S + dt B x^T;   y = S^T C + D x;   dt = softplus(W_dt h + dt_bias),
+
+    * one input projection whose rows are laid out [z: inner | x: inner | B: groups * state | C: groups * state |
+      dt: heads], inner = heads * vdim; x, B and C together pass a causal depthwise convolution over time (``taps``
+      taps with bias, the last one the current token's, zeros before the request's start) and SiLU; head h reads the B
+      and C of group h // (heads / groups);
+    * the output: y * silu(z), RMS-normed in ``norm_groups`` equal parts of the row, times ``norm``, then W_o.
+
+    What is carried from token to token, the state of a request, is S and the last ``taps - 1`` inputs of the
+    convolution, all float32: one row of the state tensor, [taps - 1][conv channels] followed by [heads][vdim][state].
+    Step sizes, decays, the convolution and the recurrence are float32 in both dtypes; the projections run in the
+    activation dtype with float32 sums and leave unrounded.
+
+    Tensors: ``in`` [2 inner + 2 groups state + heads, width], ``conv`` [channels, taps], ``conv.b`` [channels],
+    ``dt_bias``, ``A_log``, ``D`` [heads], ``norm`` [inner], ``o`` [width, inner].
+    """
+
+    def __init__(self, width: int, heads: int, groups: int, vdim: int, state: int, taps: int, norm_groups: int,
+                 norm_eps: float):
+        if heads % groups:
+            raise ValueError(f"{heads} heads cannot be grouped over {groups} groups of B and C")
+        if not 0 < state <= 256:
+            raise ValueError(f"state size {state} is not supported: the recurrence's kernel takes up to 256")
+        if not 1 <= taps <= 64:
+            raise ValueError("the convolution takes 1 to 64 taps")
+        self.width, self.heads, self.groups, self.vdim, self.n = int(width), int(heads), int(groups), int(vdim), int(state)
+        self.taps, self.norm_groups, self.norm_eps = int(taps), int(norm_groups), float(norm_eps)
+        self.inner = self.heads * self.vdim
+        if self.inner % self.norm_groups:
+            raise ValueError(f"{norm_groups} norm groups do not divide the inner width {self.inner}")
+        self.channels = self.inner + 2 * self.groups * self.n
+        self.off_z, self.off_x, self.off_dt = 0, self.inner, self.inner + self.channels
+        self.w_in = self.w_o = self.w_o_tiled = None
+        self.taps_w = self.conv_b = self.a_log = self.dt_bias = self.d_skip = self.norm_w = None
+
+    def graph_safe(self) -> bool:
+        return True     # the kernels take entries, slots and lengths from the step's device tensors
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        w, h = self.width, self.heads
+        return {"in": WeightSpec((self.off_dt + h, w), std=0.05), "conv": WeightSpec((self.channels, self.taps), std=0.5),
+                "conv.b": WeightSpec((self.channels,), std=0.1), "dt_bias": WeightSpec((h,), std=1.0, mean=-1.0),
+                "A_log": WeightSpec((h,), std=0.5, mean=-0.5), "D": WeightSpec((h,), std=0.5, mean=1.0),
+                "norm": WeightSpec((self.inner,), "norm"), "o": WeightSpec((w, self.inner))}
+
+    def state_spec(self) -> StateSpec:
+        return StateSpec(((self.taps - 1) * self.channels + self.heads * self.vdim * self.n,), "float32")
+
+    def load(self, get, device, act_dtype) -> None:
+        w_in = get("in").to(device)
+        pad = (-w_in.shape[0]) % 64      # whole tiles for the matrix-core products
+        if pad:
+            w_in = torch.cat([w_in, torch.zeros((pad, self.width), dtype=w_in.dtype, device=device)], dim=0)
+        self.w_in = w_in.contiguous()
+        self.w_o = get("o").to(device).contiguous()
+        f32 = dict(device=device, dtype=torch.float32)
+        self.taps_w, self.conv_b = get("conv").to(**f32).contiguous(), get("conv.b").to(**f32).contiguous()
+        self.a_log, self.dt_bias = get("A_log").to(**f32).contiguous(), get("dt_bias").to(**f32).contiguous()
+        self.d_skip, self.norm_w = get("D").to(**f32).contiguous(), get("norm").to(**f32).contiguous()
+        self.w_o_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_o.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            self.w_o_tiled = gemm_bf16.tile_copies_resid(self.w_o)
+
+    def device_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_o))
+
+    def forward(self, x, ctx, cache):
+        state = cache.state
+        dims = (self.heads, self.groups, self.vdim, self.n, self.taps)
+        proj = linear(x, self.w_in, torch.float32)
+        xbc, dt, decay = ops.ssd_prepare(proj, (self.off_z, self.off_x, self.off_dt), *dims, ctx.token_seq, ctx.q_start,
+                                         ctx.state_slots, state, self.taps_w, self.conv_b, self.dt_bias, self.a_log)
+        ops.ssd_conv_state(proj, self.off_x, *dims, ctx.q_start, ctx.state_slots, state)
+        y = ops.ssd_scan(xbc, dt, decay, self.d_skip, *dims, ctx.q_start, ctx.state_slots, state)
+        u = ops.ssd_out(y, proj, self.off_z, self.norm_w, self.norm_eps, self.norm_groups, x.dtype)
+        return linear_delta(u, self.w_o, None, self.w_o_tiled)
+
+
 register_mixer("gated_delta_rule", GatedDeltaRule)
+register_mixer("state_space_duality", StateSpaceDuality)

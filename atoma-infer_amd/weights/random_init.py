@@ -38,6 +38,10 @@ def random_tensor(name: str, ws: WeightSpec, seed: int, dtype: torch.dtype, norm
         t = torch.ones(ws.drawn_shape, dtype=torch.float32)
         if norm_jitter:
             t += torch.randn(ws.drawn_shape, generator=g, dtype=torch.float32) * norm_jitter
+    elif ws.init == "norm_zero":       # a norm's weight stored around zero (the part adds 1)
+        t = torch.zeros(ws.drawn_shape, dtype=torch.float32)
+        if norm_jitter:
+            t += torch.randn(ws.drawn_shape, generator=g, dtype=torch.float32) * norm_jitter
     elif ws.init == "int_table":
         return torch.randint(0, max(ws.high, 1), ws.drawn_shape, generator=g, dtype=torch.int32)
     else:
