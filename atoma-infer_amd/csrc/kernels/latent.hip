@@ -85,6 +85,59 @@ head_linear_kernel(const TA* __restrict__ x, int ldx, const TW* __restrict__ w, 
   }
 }
 
+// The same on the matrix cores for bfloat16 operands (v_mfma_f32_16x16x32_bf16, float32 sums): a workgroup takes 64
+// tokens x 64 outputs of one head, a wave 16 of the outputs against all 64 tokens; both operands' fragments come
+// straight from memory (K is a head's width: a few steps).  K a multiple of 8; a last step shorter than 32 columns is
+// filled with zeros.  The MFMA's result holds, per lane, token (lane % 16) and outputs (lane / 16) * 4 .. + 3.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+template <typename TO>
+__global__ void __launch_bounds__(256)
+head_linear_mfma_kernel(const uint16_t* __restrict__ x, int ldx, const uint16_t* __restrict__ w, TO* __restrict__ out,
+                        int ldo, const float* __restrict__ gate, int T, int H, int K, int N) {
+  const int h = blockIdx.z, n0 = blockIdx.x * 64, t0 = blockIdx.y * 64;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int msub = min(4, (T - t0 + 15) >> 4);
+  int n = n0 + wave * 16 + r16;
+  if (n > N - 1) n = N - 1;                                  // clamped rows are computed and never stored
+  const uint16_t* wp = w + ((size_t)h * N + n) * K + kg * 8;
+  const uint16_t* xp[4];
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    int t = t0 + m * 16 + r16;
+    if (t > T - 1) t = T - 1;
+    xp[m] = x + (size_t)t * ldx + (size_t)h * K + kg * 8;
+  }
+  f32x4 acc[4];
+#pragma unroll
+  for (int m = 0; m < 4; ++m) acc[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bool in = k0 + kg * 8 < K;
+    const bf16x8 wf = in ? *reinterpret_cast<const bf16x8*>(wp + k0) : zero;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      if (m < msub) {
+        const bf16x8 xf = in ? *reinterpret_cast<const bf16x8*>(xp[m] + k0) : zero;
+        acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf, acc[m], 0, 0, 0);
+      }
+    }
+  }
+  const int nb = n0 + wave * 16 + kg * 4;
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    const int t = t0 + m * 16 + r16;
+    if (m >= msub || t >= T) continue;
+    const float s = gate ? gate[(size_t)t * H + h] : 1.0f;
+    TO* dst = out + (size_t)t * ldo + (size_t)h * N + nb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (nb + i < N) dst[i] = from_f32<TO>(acc[m][i] * s);
+  }
+}
+
 extern "C" int atoma_latent_prepare(const float* proj, int ldp, int off_q, int off_c, int off_g, int nq, int rank,
                                     int rank_p, int heads, const float* w_norm, float eps, void* kcache, void* vcache,
                                     int cache_dtype, const int32_t* slot_mapping, int page_size, void* q_out,
@@ -109,6 +162,20 @@ extern "C" int atoma_head_linear(const void* x, int x_dtype, int ldx, const void
                                  hipStream_t stream) {
   if (T <= 0) return 0;
   if (H <= 0 || K <= 0 || N <= 0 || ldx < H * K || ldo < H * N || H > 65535 || (T + 15) / 16 > 65535) return ATOMA_ERR_SHAPE;
+  if (x_dtype == kBF16 && w_dtype == kBF16 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x & 15) == 0 &&
+      ((uintptr_t)w & 15) == 0 && (T + 63) / 64 <= 65535) {
+    dim3 mgrid((N + 63) / 64, (T + 63) / 64, H);
+    if (out_dtype == kBF16)
+      hipLaunchKernelGGL((head_linear_mfma_kernel<bf16_t>), mgrid, dim3(256), 0, stream, (const uint16_t*)x, ldx,
+                         (const uint16_t*)w, (bf16_t*)out, ldo, gate, T, H, K, N);
+    else if (out_dtype == kF32)
+      hipLaunchKernelGGL((head_linear_mfma_kernel<float>), mgrid, dim3(256), 0, stream, (const uint16_t*)x, ldx,
+                         (const uint16_t*)w, (float*)out, ldo, gate, T, H, K, N);
+    else
+      return ATOMA_ERR_DTYPE;
+    ATOMA_LAUNCH_CHECK();
+    return 0;
+  }
   dim3 grid((N + 63) / 64, (T + 15) / 16, H), block(256);
 #define ATOMA_HL(TA, TW, TO)                                                                                  \
   hipLaunchKernelGGL((head_linear_kernel<TA, TW, TO>), grid, block, 0, stream, (const TA*)x, ldx, (const TW*)w, \

@@ -16,6 +16,8 @@ measured by small probes, stand beside the published peaks (which stay the yards
 experts) at layer sizes that resemble a real model's, beside the Llama of equal width, heads and active feed-forward
 width: prefill of 2,048 tokens and decode steps at batch 1, 8 and 64 through the same engine, ONE line of its own
 (``--sizes 1b|3b`` picks the pair, ``--layers`` how many layers of each, 4 by default; ``--only`` one of the two).
+``--compare morulix`` does the same for the Morulix decoder (latent attention, a state-space recurrence and windowed
+attention in turn, each beside a dense feed-forward, behind one pass of its loop's entry).
 
 ``--workload`` runs one of the other two workloads instead and prints ONE line of its own:
 ``serve3b``: Llama-3.2-3B sizes, 64 requests with prompt lengths uniform in [128, 4096] (seeded), 256 generated tokens
@@ -215,6 +217,47 @@ def step_bytes_somesun(cfg: dict, batch: int, ctx: float) -> float:
     return total
 
 
+def morulix_like(llama: dict, layers: int) -> dict:
+    """The Morulix configuration beside ``llama``: the same width, vocabulary and dense feed-forward; layers in turn
+    latent attention (half as many heads of twice the size over a latent of 256 numbers), a state-space recurrence
+    (inner width twice the model's, heads of 64 columns, a state of 128, one group), windowed attention with the
+    Llama's heads and a window of 1,024 keys, and the recurrence again; one pass of the loop's entry over all layers."""
+    w, nh, nkv = llama["hidden_size"], llama["num_attention_heads"], llama["num_key_value_heads"]
+    hd = w // nh
+    mlp = {"kind": "dense", "ff": llama["intermediate_size"]}
+    sc = llama["rope_scaling"]
+    att = {"type": "attention", "mlp": mlp,
+           "mixer": {"dim": hd, "heads": nh, "kv_heads": nkv, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": 1024},
+                     "rot": {"base": llama["rope_theta"], "dims": hd,
+                             "scaling": {"factor": sc["factor"], "low": sc["low_freq_factor"],
+                                         "high": sc["high_freq_factor"], "original": sc["original_max_position_embeddings"]}}}}
+    lat = {"type": "latent_attention", "mlp": mlp,
+           "mixer": {"dim": 2 * hd, "heads": nh // 2, "kv_rank": 256, "scale": (2 * hd) ** -0.5, "vdim": 2 * hd}}
+    ssm = {"type": "mamba2", "mlp": mlp,
+           "mixer": {"conv": 4, "groups": 1, "heads": 2 * w // 64, "norm_groups": 1, "state": 128, "vdim": 64}}
+    kinds = [lat, ssm, att, ssm]
+    return {"architecture": "Morulix", "layers": [kinds[i % 4] for i in range(layers)], "norm": {"eps": 1e-5},
+            "loop": {"start": 0, "stop": layers, "times": 1}, "vocab": llama["vocab_size"], "width": w,
+            "max_positions": llama["max_position_embeddings"]}
+
+
+def step_bytes_morulix(model, cfg: dict, batch: int, ctx: float) -> float:
+    """Bytes a decode step of ``batch`` requests at context ``ctx`` has to read (and, for the state, write): every
+    matrix once, each request's latents (kept once in the keys' order and once in the values'), the keys and values
+    inside its window, the recurrent state twice."""
+    total = float(model.weight_bytes())
+    for l in cfg["layers"]:
+        m = l["mixer"]
+        if l["type"] == "latent_attention":
+            total += batch * ctx * 2.0 * 2 * (-(-m["kv_rank"] // 16) * 16)
+        elif l["type"] == "attention":
+            seen = min(ctx, m["mask"]["size"]) if m.get("mask") else ctx
+            total += batch * seen * 2.0 * 2 * m["kv_heads"] * max(m["dim"], m["vdim"])
+        else:
+            total += batch * 2 * 4.0 * m["heads"] * m["vdim"] * m["state"]
+    return total
+
+
 def compare_main(args) -> int:
     import torch
     import atoma_infer_amd  # noqa: F401
@@ -223,9 +266,10 @@ def compare_main(args) -> int:
     sizes = args.sizes if args.sizes in ("1b", "3b") else "1b"
     layers = args.layers or 4
     llama = dict(dict(LLAMA_1B, **OTHER_SIZES.get(sizes, {})), num_hidden_layers=layers)
-    sun = somesun_like(llama, layers)
+    design = args.compare
+    sun = somesun_like(llama, layers) if design == "somesun" else morulix_like(llama, layers)
     out = {}
-    for name, cfg in (("llama", llama), ("somesun", sun)):
+    for name, cfg in (("llama", llama), (design, sun)):
         if args.only and args.only != name:
             continue
         log(f"{name}: building {layers} layers at {sizes} sizes (random weights) ...")
@@ -237,7 +281,12 @@ def compare_main(args) -> int:
             st = min(args.steps, 64)
             log(f"{name}: decode at batch {b} ...")
             d, ctx = decode_run(model, b, args.prompt_len, st, min(args.warmup, 4), args.context)
-            nbytes = step_bytes_somesun(sun, b, ctx) if name == "somesun" else model.weight_bytes() + kv * ctx * b
+            if name == "somesun":
+                nbytes = step_bytes_somesun(sun, b, ctx)
+            elif name == "morulix":
+                nbytes = step_bytes_morulix(model, sun, b, ctx)
+            else:
+                nbytes = model.weight_bytes() + kv * ctx * b
             res[f"decode_b{b}_tok_s"] = round(b * st / d, 1)
             res[f"decode_b{b}_ms"] = round(d / st * 1e3, 4)
             res[f"decode_b{b}_frac"] = round(nbytes / (d / st) / 1e9 / HBM_PEAK_GBS, 4)
@@ -245,12 +294,14 @@ def compare_main(args) -> int:
         del model
         torch.cuda.empty_cache()
     l = sun["layers"][0]
-    line = {"metric": f"Somesun beside Llama at {sizes} layer sizes, {layers} layers each: prefill of "
+    shown = {"left": l["mixer"]["left"], "right": l["mixer"]["right"], "mlp": l["mlp"]} if design == "somesun" else \
+        {"layers_in_turn": [{"type": x["type"], "mixer": x["mixer"]} for x in sun["layers"][:4]], "mlp": l["mlp"],
+         "loop": sun["loop"]}
+    line = {"metric": f"{design.capitalize()} beside Llama at {sizes} layer sizes, {layers} layers each: prefill of "
                       f"{args.prefill_tokens} tokens, decode at batch 1, 8, 64 ({args.prompt_len}-token prompts)",
             "unit": "tokens/s, ms a step, fraction of 8 TB/s", "n_gpus": 1, "dtype": "bf16",
             "data": "synthetic (uniform random token ids, random weights)",
-            "config": {"width": sun["width"], "vocab": sun["vocab"], "layers": layers, "left": l["mixer"]["left"],
-                       "right": l["mixer"]["right"], "mlp": l["mlp"],
+            "config": {"width": sun["width"], "vocab": sun["vocab"], "layers": layers, **shown,
                        "llama": {k: llama[k] for k in ("hidden_size", "intermediate_size", "num_attention_heads",
                                                         "num_key_value_heads")}},
             **out}
@@ -312,9 +363,9 @@ def main() -> int:
     ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--workload", choices=["decode", *WORKLOADS], default="decode",
                     help="decode: the default run; serve3b, long8b: the other two workloads, one line of their own")
-    ap.add_argument("--compare", choices=["somesun"], default=None,
+    ap.add_argument("--compare", choices=["somesun", "morulix"], default=None,
                     help="measure that design at --sizes (1b, 3b) beside the Llama of equal sizes, one line of its own")
-    ap.add_argument("--only", choices=["llama", "somesun"], default=None, help="with --compare: one of the two models")
+    ap.add_argument("--only", choices=["llama", "somesun", "morulix"], default=None, help="with --compare: one of the two models")
     ap.add_argument("--requests", type=int, default=0, help="requests of a --workload run (default: the workload's)")
     ap.add_argument("--no-peaks", action="store_true", help="skip the probes of what the GPU delivers")
     ap.add_argument("--chain-floors", action="store_true",

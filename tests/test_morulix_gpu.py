@@ -137,7 +137,7 @@ def test_a_product_of_its_own_per_head(t, h, k, n, dtype):
     got = ops.head_linear(x.to(DEV, dtype), w.to(DEV, torch.bfloat16), dtype, gate.to(DEV))
     assert _rel(got.float().cpu().view(t, h, n), want * gate.double()[:, :, None]) < (1e-6 if dtype is torch.float32 else 5e-3)
     # rows of a wider tensor
-    wide = torch.zeros(t, h * k + 9, dtype=dtype, device=DEV)
+    wide = torch.zeros(t, h * k + 16, dtype=dtype, device=DEV)
     wide[:, : h * k] = x.to(DEV, dtype)
     assert torch.equal(ops.head_linear(wide[:, : h * k], w.to(DEV, torch.bfloat16), dtype, gate.to(DEV)), got)
 

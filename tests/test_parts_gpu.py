@@ -253,7 +253,9 @@ def test_part_registries():
     with pytest.raises(ValueError):
         make_part("mixer", "attention", width=64, num_heads=4, num_kv_heads=3, head_size=16)
     with pytest.raises(ValueError):
-        make_part("mixer", "attention", width=40, num_heads=4, num_kv_heads=4, head_size=10)   # head size refused
+        make_part("mixer", "attention", width=40, num_heads=4, num_kv_heads=4, head_size=264)   # head size refused
+    # a head size that is no multiple of 8 runs as the next multiple of 16, with zeros in the added columns
+    assert make_part("mixer", "attention", width=40, num_heads=4, num_kv_heads=4, head_size=10).hd == 16
 
 
 # ----------------------------------------------------------------------------------------------------------
