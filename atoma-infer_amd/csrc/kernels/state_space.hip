@@ -11,6 +11,8 @@
 //   ssd_scan         per (request, head, 16 columns of S): the recurrence over the entry's tokens in order, S read from
 //                    the request's state slot before and written back after.  A column of S lives in the registers of
 //                    16 neighbouring lanes (n / 16 rows each, rounded up); the tokens' inputs pass LDS in blocks;
+//   ssd_chunk        the same recurrence for entries of many tokens (prompts and their portions), 64 tokens at a time on
+//                    the matrix cores in float32 (v_mfma_f32_16x16x4_f32), see below;
 //   ssd_out          per token and norm group: y * silu(z), divided by the root mean square of its group, times the
 //                    weight, in the activation dtype.
 // The order of every sum depends on the sizes alone, so a token's result does not depend on how the request was cut
@@ -100,12 +102,12 @@ __global__ void __launch_bounds__(256)
 ssd_scan_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, const float* __restrict__ decay,
                 const float* __restrict__ d_skip, SsdShape sh, const int32_t* __restrict__ q_start,
                 const int32_t* __restrict__ state_slots, float* __restrict__ state, size_t state_stride,
-                float* __restrict__ y) {
+                float* __restrict__ y, int below) {
   __shared__ float sb[kScanTokens][16 * R], sc[kScanTokens][16 * R];
   __shared__ float sx[kScanTokens][kScanCols], sdt[kScanTokens], sa[kScanTokens];
   const int e = blockIdx.z, h = blockIdx.y, v0 = blockIdx.x * kScanCols;
   const int first = q_start[e], count = q_start[e + 1] - first;
-  if (count <= 0) return;
+  if (count <= 0 || count >= below) return;      // (entries of `below` tokens or more are the chunk kernel's)
   const int col = threadIdx.x >> 4, l = threadIdx.x & 15;
   const int v = v0 + col;
   const bool live = v < sh.vdim;
@@ -156,6 +158,154 @@ ssd_scan_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, con
       const int row = l + 16 * r;
       if (row < sh.n) s_ptr[row] = s[r];
     }
+  }
+}
+
+// The recurrence 64 tokens at a time.  With c_t the sum of the log decays of the chunk's tokens up to t (inclusive),
+//   y_t = sum_{s <= t} exp(c_t - c_s) dt_s (C_t . B_s) x_s  +  exp(c_t) S_0^T C_t  +  D x_t,
+//   S_64 = exp(c_63) S_0 + sum_s exp(c_63 - c_s) dt_s B_s x_s^T,
+// every exponent at most zero.  A workgroup owns (entry, head, 16 columns of S) and walks the entry's chunks in order;
+// per chunk its four waves make M[t][s] = (C_t . B_s) exp(c_t - c_s) dt_s for s <= t (ten tiles of 16 x 16 shared out
+// among them, into LDS), then each takes 16 tokens of y = M X + diag(exp(c)) C S, then each its share of the rows of S.
+// All products are float32 MFMAs (A operand: lane l gives A[l % 16][4 k + l / 16], B operand B[4 k + l / 16][l % 16],
+// result D[4 (l / 16) + i][l % 16]); B, C, x of the chunk, M and S wait in LDS with row strides that keep the lanes of
+// a load on different banks.  An entry's result depends on its own length and sizes alone.
+constexpr int kChunk = 64;
+constexpr int kChunkLdx = 20;       // row stride of the x tile and of S in LDS
+constexpr int kChunkLdm = kChunk + 2;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+__host__ __device__ constexpr int chunk_lds_floats(int nb) {
+  return 2 * kChunk * (16 * nb + 2) + kChunk * kChunkLdx + kChunk * kChunkLdm + 16 * nb * kChunkLdx + 4 * kChunk;
+}
+
+template <int NB>      // blocks of 16 rows of S (the state size rounded up)
+__global__ void __launch_bounds__(256)
+ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, const float* __restrict__ a_log,
+                 const float* __restrict__ d_skip, SsdShape sh, const int32_t* __restrict__ q_start,
+                 const int32_t* __restrict__ state_slots, float* __restrict__ state, size_t state_stride,
+                 float* __restrict__ y, int at_least) {
+  constexpr int NP = 16 * NB, LDN = NP + 2;
+  extern __shared__ float lds[];
+  float* Bs = lds;                         // [kChunk][LDN]
+  float* Cs = Bs + kChunk * LDN;           // [kChunk][LDN]
+  float* Xs = Cs + kChunk * LDN;           // [kChunk][kChunkLdx]
+  float* Ms = Xs + kChunk * kChunkLdx;     // [kChunk][kChunkLdm]
+  float* Ss = Ms + kChunk * kChunkLdm;     // [NP][kChunkLdx]
+  float* cum = Ss + NP * kChunkLdx;        // [kChunk] log decays summed up to each token
+  float* dts = cum + kChunk;               // [kChunk]
+  float* wts = dts + kChunk;               // [kChunk] exp(c_last - c_s) dt_s
+  float* ect = wts + kChunk;               // [kChunk] exp(c_t)
+  const int e = blockIdx.z, h = blockIdx.y, v0 = blockIdx.x * 16;
+  const int first = q_start[e], count = q_start[e + 1] - first;
+  if (count < at_least) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int inner = sh.heads * sh.vdim, gn = sh.groups * sh.n, channels = inner + 2 * gn;
+  const int g = h / (sh.heads / sh.groups);
+  const int vlive = min(16, sh.vdim - v0);
+  float* s_ptr = state + (size_t)state_slots[e] * state_stride + (size_t)(sh.taps - 1) * channels +
+                 ((size_t)h * sh.vdim + v0) * sh.n;
+  for (int idx = tid; idx < NP * 16; idx += 256) {
+    const int v = idx / NP, n = idx % NP;
+    Ss[n * kChunkLdx + v] = (v < vlive && n < sh.n) ? s_ptr[(size_t)v * sh.n + n] : 0.f;
+  }
+  const float rate = expf(a_log[h]), dh = d_skip[h];
+  for (int t0 = 0; t0 < count; t0 += kChunk) {
+    const int nt = min(kChunk, count - t0);
+    const size_t tok0 = (size_t)(first + t0);
+    __syncthreads();       // the chunk before is done with every tile
+    for (int idx = tid; idx < kChunk * NP; idx += 256) {
+      const int tt = idx / NP, n = idx % NP;
+      const bool in = tt < nt && n < sh.n;
+      const size_t base = (tok0 + tt) * channels + inner + (size_t)g * sh.n + n;
+      Bs[tt * LDN + n] = in ? xbc[base] : 0.f;
+      Cs[tt * LDN + n] = in ? xbc[base + gn] : 0.f;
+    }
+    for (int idx = tid; idx < kChunk * 16; idx += 256) {
+      const int tt = idx >> 4, v = idx & 15;
+      Xs[tt * kChunkLdx + v] = (tt < nt && v < vlive) ? xbc[(tok0 + tt) * channels + (size_t)h * sh.vdim + v0 + v] : 0.f;
+    }
+    if (tid < kChunk) dts[tid] = tid < nt ? dt[(tok0 + tid) * sh.heads + h] : 0.f;
+    __syncthreads();
+    if (wave == 0) {
+      // inclusive sums of the log decays over the 64 lanes
+      float c = -rate * dts[lane];
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const float up = __shfl_up(c, o, 64);
+        if (lane >= o) c += up;
+      }
+      cum[lane] = c;
+      const float last = __shfl(c, 63, 64);
+      wts[lane] = expf(last - c) * dts[lane];
+      ect[lane] = expf(c);
+    }
+    __syncthreads();
+    // M: the ten tiles on and below the diagonal, dealt to the waves in turn
+    {
+      int j = 0;
+      for (int tb = 0; tb < 4; ++tb)
+        for (int sb = 0; sb <= tb; ++sb, ++j) {
+          if ((j & 3) != wave) continue;
+          f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+          const float* cp = Cs + (tb * 16 + r16) * LDN + kg;
+          const float* bp = Bs + (sb * 16 + r16) * LDN + kg;
+#pragma unroll 8
+          for (int k = 0; k < NP; k += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(cp[k], bp[k], acc, 0, 0, 0);
+          const int s = sb * 16 + r16;
+          const float cs = cum[s], ds = dts[s];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int t = tb * 16 + 4 * kg + i;
+            Ms[t * kChunkLdm + s] = s <= t ? acc[i] * expf(cum[t] - cs) * ds : 0.f;
+          }
+        }
+    }
+    __syncthreads();
+    // y of the wave's 16 tokens
+    if (wave * 16 < nt) {
+      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+      const int tb = wave;
+      const float* mp = Ms + (tb * 16 + r16) * kChunkLdm + kg;
+      const float* xp = Xs + kg * kChunkLdx + r16;
+      for (int k = 0; k < (tb + 1) * 16; k += 4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(mp[k], xp[k * kChunkLdx], acc, 0, 0, 0);
+      const float et = ect[tb * 16 + r16];
+      const float* cp = Cs + (tb * 16 + r16) * LDN + kg;
+      const float* sp = Ss + kg * kChunkLdx + r16;
+#pragma unroll 8
+      for (int k = 0; k < NP; k += 4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(et * cp[k], sp[k * kChunkLdx], acc, 0, 0, 0);
+      if (r16 < vlive) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int t = tb * 16 + 4 * kg + i;
+          if (t < nt) y[(tok0 + t) * inner + (size_t)h * sh.vdim + v0 + r16] = acc[i] + dh * Xs[t * kChunkLdx + r16];
+        }
+      }
+    }
+    __syncthreads();       // every wave has read S
+    {
+      const float keep = ect[kChunk - 1];
+      for (int nb = wave; nb < NB; nb += 4) {
+        f32x4 acc;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = keep * Ss[(nb * 16 + 4 * kg + i) * kChunkLdx + r16];
+        const float* bp = Bs + kg * LDN + nb * 16 + r16;
+        const float* xp = Xs + kg * kChunkLdx + r16;
+#pragma unroll 8
+        for (int k = 0; k < kChunk; k += 4)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(bp[k * LDN] * wts[k + kg], xp[k * kChunkLdx], acc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) Ss[(nb * 16 + 4 * kg + i) * kChunkLdx + r16] = acc[i];
+      }
+    }
+  }
+  __syncthreads();
+  for (int idx = tid; idx < NP * 16; idx += 256) {
+    const int v = idx / NP, n = idx % NP;
+    if (v < vlive && n < sh.n) s_ptr[(size_t)v * sh.n + n] = Ss[n * kChunkLdx + v];
   }
 }
 
@@ -220,7 +370,7 @@ extern "C" int atoma_ssd_conv_state(const float* proj, int ldp, int off_x, int h
 extern "C" int atoma_ssd_scan(const float* xbc, const float* dt, const float* decay, const float* d_skip, int heads,
                               int groups, int vdim, int n, int taps, const int32_t* q_start,
                               const int32_t* state_slots, float* state, size_t state_stride, float* y,
-                              int n_entries, hipStream_t stream) {
+                              int n_entries, int below, hipStream_t stream) {
   if (n_entries <= 0) return 0;
   SsdShape sh{heads, groups, vdim, n, taps, 1, 0, 0, 0};
   if (!shape_ok(sh) || n_entries > 65535 || heads > 65535) return ATOMA_ERR_SHAPE;
@@ -228,7 +378,7 @@ extern "C" int atoma_ssd_scan(const float* xbc, const float* dt, const float* de
   const int rows = (n + 15) / 16;
 #define ATOMA_SCAN(R)                                                                                              \
   hipLaunchKernelGGL((ssd_scan_kernel<R>), grid, block, 0, stream, xbc, dt, decay, d_skip, sh, q_start, state_slots, \
-                     state, state_stride, y)
+                     state, state_stride, y, below)
   if (rows <= 1) ATOMA_SCAN(1);
   else if (rows <= 2) ATOMA_SCAN(2);
   else if (rows <= 3) ATOMA_SCAN(3);
@@ -238,6 +388,51 @@ extern "C" int atoma_ssd_scan(const float* xbc, const float* dt, const float* de
   else if (rows <= 12) ATOMA_SCAN(12);
   else ATOMA_SCAN(16);
 #undef ATOMA_SCAN
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+// The largest state size the chunk kernel takes (its tiles of B and C must fit the CU's LDS beside the rest).
+extern "C" int atoma_ssd_chunk_max_state() { return 128; }
+
+template <int NB>
+static int launch_chunk(dim3 grid, hipStream_t stream, const float* xbc, const float* dt, const float* a_log,
+                        const float* d_skip, const SsdShape& sh, const int32_t* q_start, const int32_t* state_slots,
+                        float* state, size_t state_stride, float* y, int at_least) {
+  const size_t bytes = (size_t)chunk_lds_floats(NB) * sizeof(float);
+  static bool asked = false;      // (per instantiation) more than the default 64 KB of LDS
+  if (!asked && bytes > 64 * 1024) {
+    hipError_t err = hipFuncSetAttribute((const void*)ssd_chunk_kernel<NB>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)bytes);
+    if (err != hipSuccess) return (int)err;
+    asked = true;
+  }
+  hipLaunchKernelGGL((ssd_chunk_kernel<NB>), grid, dim3(256), bytes, stream, xbc, dt, a_log, d_skip, sh, q_start,
+                     state_slots, state, state_stride, y, at_least);
+  return 0;
+}
+
+// entries of at least `at_least` tokens; the others are left to atoma_ssd_scan(below = at_least)
+extern "C" int atoma_ssd_chunk(const float* xbc, const float* dt, const float* a_log, const float* d_skip, int heads,
+                               int groups, int vdim, int n, int taps, const int32_t* q_start,
+                               const int32_t* state_slots, float* state, size_t state_stride, float* y,
+                               int n_entries, int at_least, hipStream_t stream) {
+  if (n_entries <= 0) return 0;
+  SsdShape sh{heads, groups, vdim, n, taps, 1, 0, 0, 0};
+  if (!shape_ok(sh) || n > 128 || n_entries > 65535 || heads > 65535 || at_least < 1) return ATOMA_ERR_SHAPE;
+  dim3 grid((vdim + 15) / 16, heads, n_entries);
+  int rc;
+  switch ((n + 15) / 16) {
+    case 1: rc = launch_chunk<1>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
+    case 2: rc = launch_chunk<2>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
+    case 3: rc = launch_chunk<3>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
+    case 4: rc = launch_chunk<4>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
+    case 5: rc = launch_chunk<5>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
+    case 6: rc = launch_chunk<6>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
+    case 7: rc = launch_chunk<7>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
+    default: rc = launch_chunk<8>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
+  }
+  if (rc != 0) return rc;
   ATOMA_LAUNCH_CHECK();
   return 0;
 }

@@ -538,24 +538,42 @@ def ssd_conv_state(proj: torch.Tensor, off_x: int, heads: int, groups: int, vdim
         ctypes.c_size_t(state.stride(0)), s, _stream()), "ssd_conv_state")
 
 
-def ssd_scan(xbc: torch.Tensor, dt: torch.Tensor, decay: torch.Tensor, d_skip: torch.Tensor, heads: int, groups: int,
-             vdim: int, n: int, taps: int, q_start: torch.Tensor, state_slots: torch.Tensor,
-             state: torch.Tensor) -> torch.Tensor:
+SSD_CHUNK_MIN_TOKENS = 16      # entries of at least this many tokens run 64 tokens at a time on the matrix cores
+
+
+def ssd_scan(xbc: torch.Tensor, dt: torch.Tensor, decay: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor,
+             heads: int, groups: int, vdim: int, n: int, taps: int, q_start: torch.Tensor,
+             state_slots: torch.Tensor, state: torch.Tensor, counts=None) -> torch.Tensor:
     """The recurrence over every entry's tokens, from and into the requests' state rows; returns y float32
-    [T, heads vdim] = S^T C + D x."""
-    _dev(xbc, dt, decay, d_skip, q_start, state_slots, state)
+    [T, heads vdim] = S^T C + D x.  ``counts``: the entries' numbers of tokens on the host; with them, entries of
+    ``SSD_CHUNK_MIN_TOKENS`` tokens or more (and a state of at most 128) are worked 64 tokens at a time by float32
+    MFMAs, the others token by token.  Which of the two an entry gets depends on its own length alone."""
+    _dev(xbc, dt, decay, a_log, d_skip, q_start, state_slots, state)
     t, s = xbc.shape[0], state_slots.numel()
     channels = _ssd_state_ok(state, heads, groups, vdim, n, taps)
     _need(xbc.dtype is torch.float32 and xbc.is_contiguous() and tuple(xbc.shape) == (t, channels), "xbc: bad shape")
     for x, what in ((dt, "dt"), (decay, "decay")):
         _need(x.dtype is torch.float32 and x.is_contiguous() and tuple(x.shape) == (t, heads), f"{what}: bad shape")
     _f32(d_skip, "D", heads)
+    _f32(a_log, "A_log", heads)
     _i32(q_start, "q_start", s + 1)
     _i32(state_slots, "state_slots", s)
     y = torch.empty((t, heads * vdim), dtype=torch.float32, device=xbc.device)
-    _check(_module("state_space").atoma_ssd_scan(
-        _p(xbc), _p(dt), _p(decay), _p(d_skip), heads, groups, vdim, n, taps, _p(q_start), _p(state_slots), _p(state),
-        ctypes.c_size_t(state.stride(0)), _p(y), s, _stream()), "ssd_scan")
+    lib = _module("state_space")
+    longest = shortest = 0
+    if counts is not None and len(counts) and n <= lib.atoma_ssd_chunk_max_state():
+        _need(len(counts) == s, "one count per entry")
+        longest, shortest = int(max(counts)), int(min(counts))
+    below = 1 << 30
+    if longest >= SSD_CHUNK_MIN_TOKENS:
+        below = SSD_CHUNK_MIN_TOKENS
+        _check(lib.atoma_ssd_chunk(
+            _p(xbc), _p(dt), _p(a_log), _p(d_skip), heads, groups, vdim, n, taps, _p(q_start), _p(state_slots), _p(state),
+            ctypes.c_size_t(state.stride(0)), _p(y), s, below, _stream()), "ssd_chunk")
+    if shortest < below:
+        _check(lib.atoma_ssd_scan(
+            _p(xbc), _p(dt), _p(decay), _p(d_skip), heads, groups, vdim, n, taps, _p(q_start), _p(state_slots), _p(state),
+            ctypes.c_size_t(state.stride(0)), _p(y), s, below, _stream()), "ssd_scan")
     return y
 
 

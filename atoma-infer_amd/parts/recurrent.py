@@ -205,7 +205,8 @@ class StateSpaceDuality(Mixer):
         xbc, dt, decay = ops.ssd_prepare(proj, (self.off_z, self.off_x, self.off_dt), *dims, ctx.token_seq, ctx.q_start,
                                          ctx.state_slots, state, self.taps_w, self.conv_b, self.dt_bias, self.a_log)
         ops.ssd_conv_state(proj, self.off_x, *dims, ctx.q_start, ctx.state_slots, state)
-        y = ops.ssd_scan(xbc, dt, decay, self.d_skip, *dims, ctx.q_start, ctx.state_slots, state)
+        y = ops.ssd_scan(xbc, dt, decay, self.a_log, self.d_skip, *dims, ctx.q_start, ctx.state_slots, state,
+                         counts=ctx.h_counts)
         u = ops.ssd_out(y, proj, self.off_z, self.norm_w, self.norm_eps, self.norm_groups, x.dtype)
         return linear_delta(u, self.w_o, None, self.w_o_tiled)
 

@@ -146,17 +146,20 @@ def test_a_product_of_its_own_per_head(t, h, k, n, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads, groups, vdim, n, taps, parts", [(4, 2, 16, 16, 3, 2), (3, 1, 8, 12, 2, 1), (2, 2, 40, 100, 5, 5),
-                                                                 (1, 1, 5, 1, 1, 5), (6, 3, 24, 200, 4, 3), (4, 4, 64, 48, 4, 2)])
+                                                                 (1, 1, 5, 1, 1, 5), (6, 3, 24, 200, 4, 3), (4, 4, 64, 48, 4, 2),
+                                                                 (2, 1, 32, 128, 4, 1)])
 def test_state_space_recurrence_alone_whole_and_in_portions(heads, groups, vdim, n, taps, parts, dtype):
     """The mixer on hand-made steps: two requests side by side, cut into portions of unequal lengths (one token, two,
-    fewer than the convolution has taps, many), each carried by its state slot; against the plain recurrence."""
+    fewer than the convolution has taps, many), each carried by its state slot; against the plain recurrence.  Portions
+    of 16 tokens and more run 64 tokens at a time on the matrix cores (states up to 128), shorter ones token by token:
+    the portions here are of both kinds, side by side in one step too, with chunks that are full and that are not."""
     from atoma_infer_amd.parts import StateSpaceDuality
     width = 64
     part = StateSpaceDuality(width, heads, groups, vdim, n, taps, parts, 1e-5)
     w = _drawn(part, "x.", 5, boost=(("in", 8),))
     _load(part, w, dtype)
     g = torch.Generator().manual_seed(n)
-    lens = (37, 9)
+    lens = (267, 29)
     hs = [torch.randn(c, width, generator=g).to(torch.bfloat16).float() for c in lens]
     m = {"heads": heads, "groups": groups, "vdim": vdim, "state": n, "conv": taps, "norm_groups": parts}
     want = [pm.mamba2(h.double(), {"r." + k: v.double() for k, v in w.items()}, "r.", m, 1e-5) for h in hs]
@@ -164,7 +167,8 @@ def test_state_space_recurrence_alone_whole_and_in_portions(heads, groups, vdim,
     state[1].fill_(7.0)                       # another request's slot must stay as it is
     cache = types.SimpleNamespace(state=state)
     got, at = [[], []], [0, 0]
-    for cuts in ([(0, 1), (1, 2)], [(0, 2)], [(1, 1), (0, 1)], [(0, 30), (1, 6)], [(0, 3)]):
+    for cuts in ([(0, 1), (1, 2)], [(0, 2)], [(1, 1), (0, 1)], [(0, 30), (1, 6)], [(0, 3)], [(0, 64), (1, 17)], [(0, 150)],
+                 [(0, 16), (1, 3)]):
         ctx = _ctx([at[r] for r, _ in cuts], [c for _, c in cuts], [3 if r == 0 else 0 for r, _ in cuts])
         x = torch.cat([hs[r][at[r]: at[r] + c] for r, c in cuts]).to(DEV, dtype)
         y = _flat(part.forward(x, ctx, cache))
