@@ -167,17 +167,20 @@ ssd_scan_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, con
 // every exponent at most zero.  A workgroup owns (entry, head, 16 columns of S) and walks the entry's chunks in order;
 // per chunk its four waves make M[t][s] = (C_t . B_s) exp(c_t - c_s) dt_s for s <= t (ten tiles of 16 x 16 shared out
 // among them, into LDS), then each takes 16 tokens of y = M X + diag(exp(c)) C S, then each its share of the rows of S.
-// All products are float32 MFMAs (A operand: lane l gives A[l % 16][4 k + l / 16], B operand B[4 k + l / 16][l % 16],
-// result D[4 (l / 16) + i][l % 16]); B, C, x of the chunk, M and S wait in LDS with row strides that keep the lanes of
-// a load on different banks.  An entry's result depends on its own length and sizes alone.
+// All products are float32 MFMAs of 16 x 16 x 4 (result D[4 (l / 16) + i][l % 16] in lane l).  The sum over k of a
+// block of 16 is taken in the order that lets a lane fetch its four values with one 16-byte load from LDS: in the
+// block's MFMA j, lane l gives A[l % 16][4 (l / 16) + j] and B[4 (l / 16) + j][l % 16]; tiles whose k runs along their
+// rows in memory (x and S) are kept transposed in LDS for it.  The next chunk's B, C, x and dt are asked for while this
+// one is worked on.  An entry's result depends on its own length and sizes alone.
 constexpr int kChunk = 64;
-constexpr int kChunkLdx = 20;       // row stride of the x tile and of S in LDS
-constexpr int kChunkLdm = kChunk + 2;
+constexpr int kChunkLdt = kChunk + 4;      // row stride of the tiles whose rows are 64 tokens long (M, x transposed)
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
 __host__ __device__ constexpr int chunk_lds_floats(int nb) {
-  return 2 * kChunk * (16 * nb + 2) + kChunk * kChunkLdx + kChunk * kChunkLdm + 16 * nb * kChunkLdx + 4 * kChunk;
+  return 2 * kChunk * (16 * nb + 4) + kChunk * kChunkLdt + 16 * kChunkLdt + 16 * (16 * nb + 4) + 4 * kChunk;
 }
+
+__device__ __forceinline__ f32x4 lds4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
 
 template <int NB>      // blocks of 16 rows of S (the state size rounded up)
 __global__ void __launch_bounds__(256)
@@ -185,14 +188,14 @@ ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, co
                  const float* __restrict__ d_skip, SsdShape sh, const int32_t* __restrict__ q_start,
                  const int32_t* __restrict__ state_slots, float* __restrict__ state, size_t state_stride,
                  float* __restrict__ y, int at_least) {
-  constexpr int NP = 16 * NB, LDN = NP + 2;
-  extern __shared__ float lds[];
-  float* Bs = lds;                         // [kChunk][LDN]
-  float* Cs = Bs + kChunk * LDN;           // [kChunk][LDN]
-  float* Xs = Cs + kChunk * LDN;           // [kChunk][kChunkLdx]
-  float* Ms = Xs + kChunk * kChunkLdx;     // [kChunk][kChunkLdm]
-  float* Ss = Ms + kChunk * kChunkLdm;     // [NP][kChunkLdx]
-  float* cum = Ss + NP * kChunkLdx;        // [kChunk] log decays summed up to each token
+  constexpr int NP = 16 * NB, LDN = NP + 4;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* Bs = lds;                         // [kChunk][LDN]   B of the chunk's tokens
+  float* Cs = Bs + kChunk * LDN;           // [kChunk][LDN]   C
+  float* Ms = Cs + kChunk * LDN;           // [kChunk][kChunkLdt]   M[t][s]
+  float* Xt = Ms + kChunk * kChunkLdt;     // [16][kChunkLdt]  x transposed: [column][token]
+  float* St = Xt + 16 * kChunkLdt;         // [16][LDN]        S transposed: [column][row], as the state keeps it
+  float* cum = St + 16 * LDN;              // [kChunk] log decays summed up to each token
   float* dts = cum + kChunk;               // [kChunk]
   float* wts = dts + kChunk;               // [kChunk] exp(c_last - c_s) dt_s
   float* ect = wts + kChunk;               // [kChunk] exp(c_t)
@@ -208,26 +211,49 @@ ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, co
                  ((size_t)h * sh.vdim + v0) * sh.n;
   for (int idx = tid; idx < NP * 16; idx += 256) {
     const int v = idx / NP, n = idx % NP;
-    Ss[n * kChunkLdx + v] = (v < vlive && n < sh.n) ? s_ptr[(size_t)v * sh.n + n] : 0.f;
+    St[v * LDN + n] = (v < vlive && n < sh.n) ? s_ptr[(size_t)v * sh.n + n] : 0.f;
   }
   const float rate = expf(a_log[h]), dh = d_skip[h];
+  // A chunk's B, C, x and dt are asked for while the chunk before is worked on, and wait in registers meanwhile.
+  constexpr int PER = kChunk * NP / 256;        // elements of a [64][NP] tile a thread moves
+  float rb[PER], rc[PER], rx[4], rdt = 0.f;
+  auto fetch = [&](int t0) {
+    const int nt = min(kChunk, count - t0);
+    const size_t tok0 = (size_t)(first + t0);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = tid + i * 256, tt = idx / NP, n = idx % NP;
+      const bool in = tt < nt && n < sh.n;
+      const size_t base = (tok0 + tt) * channels + inner + (size_t)g * sh.n + n;
+      rb[i] = in ? xbc[base] : 0.f;
+      rc[i] = in ? xbc[base + gn] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + i * 256, tt = idx >> 4, v = idx & 15;
+      rx[i] = (tt < nt && v < vlive) ? xbc[(tok0 + tt) * channels + (size_t)h * sh.vdim + v0 + v] : 0.f;
+    }
+    if (tid < kChunk) rdt = tid < nt ? dt[(tok0 + tid) * sh.heads + h] : 0.f;
+  };
+  fetch(0);
   for (int t0 = 0; t0 < count; t0 += kChunk) {
     const int nt = min(kChunk, count - t0);
     const size_t tok0 = (size_t)(first + t0);
     __syncthreads();       // the chunk before is done with every tile
-    for (int idx = tid; idx < kChunk * NP; idx += 256) {
-      const int tt = idx / NP, n = idx % NP;
-      const bool in = tt < nt && n < sh.n;
-      const size_t base = (tok0 + tt) * channels + inner + (size_t)g * sh.n + n;
-      Bs[tt * LDN + n] = in ? xbc[base] : 0.f;
-      Cs[tt * LDN + n] = in ? xbc[base + gn] : 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = tid + i * 256, tt = idx / NP, n = idx % NP;
+      Bs[tt * LDN + n] = rb[i];
+      Cs[tt * LDN + n] = rc[i];
     }
-    for (int idx = tid; idx < kChunk * 16; idx += 256) {
-      const int tt = idx >> 4, v = idx & 15;
-      Xs[tt * kChunkLdx + v] = (tt < nt && v < vlive) ? xbc[(tok0 + tt) * channels + (size_t)h * sh.vdim + v0 + v] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + i * 256;
+      Xt[(idx & 15) * kChunkLdt + (idx >> 4)] = rx[i];
     }
-    if (tid < kChunk) dts[tid] = tid < nt ? dt[(tok0 + tid) * sh.heads + h] : 0.f;
+    if (tid < kChunk) dts[tid] = rdt;
     __syncthreads();
+    if (t0 + kChunk < count) fetch(t0 + kChunk);
     if (wave == 0) {
       // inclusive sums of the log decays over the 64 lanes
       float c = -rate * dts[lane];
@@ -241,47 +267,66 @@ ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, co
       wts[lane] = expf(last - c) * dts[lane];
       ect[lane] = expf(c);
     }
-    __syncthreads();
-    // M: the ten tiles on and below the diagonal, dealt to the waves in turn
-    {
-      int j = 0;
-      for (int tb = 0; tb < 4; ++tb)
-        for (int sb = 0; sb <= tb; ++sb, ++j) {
-          if ((j & 3) != wave) continue;
-          f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-          const float* cp = Cs + (tb * 16 + r16) * LDN + kg;
-          const float* bp = Bs + (sb * 16 + r16) * LDN + kg;
-#pragma unroll 8
-          for (int k = 0; k < NP; k += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(cp[k], bp[k], acc, 0, 0, 0);
-          const int s = sb * 16 + r16;
-          const float cs = cum[s], ds = dts[s];
+    // M: the ten tiles on and below the diagonal, dealt to the waves in turn (the products need no decay yet)
+    // (tile j is the wave's (j / 4)-th; the loops are unrolled, so the tiles wait in registers named at compile time)
+    f32x4 mt[3];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int t = tb * 16 + 4 * kg + i;
-            Ms[t * kChunkLdm + s] = s <= t ? acc[i] * expf(cum[t] - cs) * ds : 0.f;
-          }
+    for (int j = 0; j < 10; ++j) {
+      const int tb = j >= 6 ? 3 : j >= 3 ? 2 : j >= 1 ? 1 : 0, sb = j - tb * (tb + 1) / 2;
+      if ((j & 3) == wave) {
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+        const float* cp = Cs + (tb * 16 + r16) * LDN + 4 * kg;
+        const float* bp = Bs + (sb * 16 + r16) * LDN + 4 * kg;
+#pragma unroll
+        for (int k = 0; k < NP; k += 16) {
+          const f32x4 a4 = lds4(cp + k), b4 = lds4(bp + k);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[q], b4[q], acc, 0, 0, 0);
         }
+        mt[j >> 2] = acc;
+      }
+    }
+    __syncthreads();       // the sums of the log decays are there
+#pragma unroll
+    for (int j = 0; j < 10; ++j) {
+      const int tb = j >= 6 ? 3 : j >= 3 ? 2 : j >= 1 ? 1 : 0, sb = j - tb * (tb + 1) / 2;
+      if ((j & 3) == wave) {
+        const f32x4 acc = mt[j >> 2];
+        const int s = sb * 16 + r16;
+        const float cs = cum[s], ds = dts[s];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int t = tb * 16 + 4 * kg + i;
+          Ms[t * kChunkLdt + s] = s <= t ? acc[i] * expf(cum[t] - cs) * ds : 0.f;
+        }
+      }
     }
     __syncthreads();
     // y of the wave's 16 tokens
     if (wave * 16 < nt) {
       f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
       const int tb = wave;
-      const float* mp = Ms + (tb * 16 + r16) * kChunkLdm + kg;
-      const float* xp = Xs + kg * kChunkLdx + r16;
-      for (int k = 0; k < (tb + 1) * 16; k += 4)
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(mp[k], xp[k * kChunkLdx], acc, 0, 0, 0);
+      const float* mp = Ms + (tb * 16 + r16) * kChunkLdt + 4 * kg;
+      const float* xp = Xt + r16 * kChunkLdt + 4 * kg;
+      for (int k = 0; k < (tb + 1) * 16; k += 16) {
+        const f32x4 a4 = lds4(mp + k), b4 = lds4(xp + k);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[q], b4[q], acc, 0, 0, 0);
+      }
       const float et = ect[tb * 16 + r16];
-      const float* cp = Cs + (tb * 16 + r16) * LDN + kg;
-      const float* sp = Ss + kg * kChunkLdx + r16;
-#pragma unroll 8
-      for (int k = 0; k < NP; k += 4)
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(et * cp[k], sp[k * kChunkLdx], acc, 0, 0, 0);
+      const float* cp = Cs + (tb * 16 + r16) * LDN + 4 * kg;
+      const float* sp = St + r16 * LDN + 4 * kg;
+#pragma unroll
+      for (int k = 0; k < NP; k += 16) {
+        const f32x4 a4 = lds4(cp + k), b4 = lds4(sp + k);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(et * a4[q], b4[q], acc, 0, 0, 0);
+      }
       if (r16 < vlive) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int t = tb * 16 + 4 * kg + i;
-          if (t < nt) y[(tok0 + t) * inner + (size_t)h * sh.vdim + v0 + r16] = acc[i] + dh * Xs[t * kChunkLdx + r16];
+          if (t < nt) y[(tok0 + t) * inner + (size_t)h * sh.vdim + v0 + r16] = acc[i] + dh * Xt[r16 * kChunkLdt + t];
         }
       }
     }
@@ -289,23 +334,28 @@ ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, co
     {
       const float keep = ect[kChunk - 1];
       for (int nb = wave; nb < NB; nb += 4) {
-        f32x4 acc;
+        // lane: rows nb * 16 + 4 (l / 16) .. + 3 of S, column l % 16: four neighbours of the transposed tile
+        float* sp = St + r16 * LDN + nb * 16 + 4 * kg;
+        f32x4 acc = lds4(sp);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] = keep * Ss[(nb * 16 + 4 * kg + i) * kChunkLdx + r16];
-        const float* bp = Bs + kg * LDN + nb * 16 + r16;
-        const float* xp = Xs + kg * kChunkLdx + r16;
-#pragma unroll 8
-        for (int k = 0; k < kChunk; k += 4)
-          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(bp[k * LDN] * wts[k + kg], xp[k * kChunkLdx], acc, 0, 0, 0);
+        for (int i = 0; i < 4; ++i) acc[i] *= keep;
+        const float* bp = Bs + (4 * kg) * LDN + nb * 16 + r16;
+        const float* xp = Xt + r16 * kChunkLdt + 4 * kg;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) Ss[(nb * 16 + 4 * kg + i) * kChunkLdx + r16] = acc[i];
+        for (int k = 0; k < kChunk; k += 16) {
+          const f32x4 w4 = lds4(wts + k + 4 * kg), b4 = lds4(xp + k);
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(bp[(k + q) * LDN] * w4[q], b4[q], acc, 0, 0, 0);
+        }
+        *reinterpret_cast<f32x4*>(sp) = acc;
       }
     }
   }
   __syncthreads();
   for (int idx = tid; idx < NP * 16; idx += 256) {
     const int v = idx / NP, n = idx % NP;
-    if (v < vlive && n < sh.n) s_ptr[(size_t)v * sh.n + n] = Ss[n * kChunkLdx + v];
+    if (v < vlive && n < sh.n) s_ptr[(size_t)v * sh.n + n] = St[v * LDN + n];
   }
 }
 
