@@ -359,24 +359,49 @@ ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, co
   }
 }
 
-// one workgroup per (token, norm group)
-template <typename TO>
+// one workgroup per (token, norm group); parts of up to 4,096 columns wait in registers between the two passes
+template <typename TO, int PER>
 __global__ void __launch_bounds__(256)
 ssd_out_kernel(const float* __restrict__ y, const float* __restrict__ proj, int ldp, int off_z,
                const float* __restrict__ w, float eps, int inner, int part, TO* __restrict__ out) {
   __shared__ float scratch[4];
   const int t = blockIdx.x, p0 = blockIdx.y * part;
+  const float* zp = proj + (size_t)t * ldp + off_z + p0;
+  const float* yp = y + (size_t)t * inner + p0;
   float ss = 0.f;
+  if constexpr (PER > 0) {
+    constexpr int P = PER > 0 ? PER : 1;
+    float u[P], yv[P], zv[P];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int i = threadIdx.x + j * 256;
+      yv[j] = i < part ? yp[i] : 0.f;
+      zv[j] = i < part ? zp[i] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      u[j] = yv[j] * (zv[j] * ssd_sigmoid(zv[j]));
+      ss = fmaf(u[j], u[j], ss);
+    }
+    ss = block_sum<4>(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)part + eps);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int i = threadIdx.x + j * 256;
+      if (i < part) out[(size_t)t * inner + p0 + i] = from_f32<TO>(u[j] * inv * w[p0 + i]);
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < part; i += 256) {
-    const float z = proj[(size_t)t * ldp + off_z + p0 + i];
-    const float u = y[(size_t)t * inner + p0 + i] * (z * ssd_sigmoid(z));
+    const float z = zp[i];
+    const float u = yp[i] * (z * ssd_sigmoid(z));
     ss = fmaf(u, u, ss);
   }
   ss = block_sum<4>(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)part + eps);
   for (int i = threadIdx.x; i < part; i += 256) {
-    const float z = proj[(size_t)t * ldp + off_z + p0 + i];
-    const float u = y[(size_t)t * inner + p0 + i] * (z * ssd_sigmoid(z));
+    const float z = zp[i];
+    const float u = yp[i] * (z * ssd_sigmoid(z));
     out[(size_t)t * inner + p0 + i] = from_f32<TO>(u * inv * w[p0 + i]);
   }
 }
@@ -493,12 +518,20 @@ extern "C" int atoma_ssd_out(const float* y, const float* proj, int ldp, int off
   if (inner <= 0 || norm_groups <= 0 || inner % norm_groups || norm_groups > 65535 || ldp < inner) return ATOMA_ERR_SHAPE;
   const int part = inner / norm_groups;
   dim3 grid(n_tokens, norm_groups), block(256);
-  if (out_dtype == kF32)
-    hipLaunchKernelGGL((ssd_out_kernel<float>), grid, block, 0, stream, y, proj, ldp, off_z, w, eps, inner, part, (float*)out);
-  else if (out_dtype == kBF16)
-    hipLaunchKernelGGL((ssd_out_kernel<bf16_t>), grid, block, 0, stream, y, proj, ldp, off_z, w, eps, inner, part, (bf16_t*)out);
-  else
-    return ATOMA_ERR_DTYPE;
+#define ATOMA_SSD_OUT(TO, PER)                                                                                    \
+  hipLaunchKernelGGL((ssd_out_kernel<TO, PER>), grid, block, 0, stream, y, proj, ldp, off_z, w, eps, inner, part, \
+                     (TO*)out)
+#define ATOMA_SSD_OUT_BY_PART(TO)                 \
+  do {                                            \
+    if (part <= 1024) ATOMA_SSD_OUT(TO, 4);       \
+    else if (part <= 4096) ATOMA_SSD_OUT(TO, 16); \
+    else ATOMA_SSD_OUT(TO, 0);                    \
+  } while (0)
+  if (out_dtype == kF32) ATOMA_SSD_OUT_BY_PART(float);
+  else if (out_dtype == kBF16) ATOMA_SSD_OUT_BY_PART(bf16_t);
+  else return ATOMA_ERR_DTYPE;
+#undef ATOMA_SSD_OUT_BY_PART
+#undef ATOMA_SSD_OUT
   ATOMA_LAUNCH_CHECK();
   return 0;
 }

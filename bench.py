@@ -219,7 +219,8 @@ def step_bytes_somesun(cfg: dict, batch: int, ctx: float) -> float:
 
 def morulix_like(llama: dict, layers: int) -> dict:
     """The Morulix configuration beside ``llama``: the same width, vocabulary and dense feed-forward; layers in turn
-    latent attention (half as many heads of twice the size over a latent of 256 numbers), a state-space recurrence
+    latent attention (half as many heads of twice the size over a latent of 128 numbers, 256 from a width of 3,072
+    on), a state-space recurrence
     (inner width twice the model's, heads of 64 columns, a state of 128, one group), windowed attention with the
     Llama's heads and a window of 1,024 keys, and the recurrence again; one pass of the loop's entry over all layers."""
     w, nh, nkv = llama["hidden_size"], llama["num_attention_heads"], llama["num_key_value_heads"]
@@ -232,7 +233,7 @@ def morulix_like(llama: dict, layers: int) -> dict:
                              "scaling": {"factor": sc["factor"], "low": sc["low_freq_factor"],
                                          "high": sc["high_freq_factor"], "original": sc["original_max_position_embeddings"]}}}}
     lat = {"type": "latent_attention", "mlp": mlp,
-           "mixer": {"dim": 2 * hd, "heads": nh // 2, "kv_rank": 256, "scale": (2 * hd) ** -0.5, "vdim": 2 * hd}}
+           "mixer": {"dim": 2 * hd, "heads": nh // 2, "kv_rank": 128 if w < 3072 else 256, "scale": (2 * hd) ** -0.5, "vdim": 2 * hd}}
     ssm = {"type": "mamba2", "mlp": mlp,
            "mixer": {"conv": 4, "groups": 1, "heads": 2 * w // 64, "norm_groups": 1, "state": 128, "vdim": 64}}
     kinds = [lat, ssm, att, ssm]
