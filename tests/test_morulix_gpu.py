@@ -147,7 +147,7 @@ def test_a_product_of_its_own_per_head(t, h, k, n, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads, groups, vdim, n, taps, parts", [(4, 2, 16, 16, 3, 2), (3, 1, 8, 12, 2, 1), (2, 2, 40, 100, 5, 5),
                                                                  (1, 1, 5, 1, 1, 5), (6, 3, 24, 200, 4, 3), (4, 4, 64, 48, 4, 2),
-                                                                 (2, 1, 32, 128, 4, 1)])
+                                                                 (2, 1, 32, 128, 4, 1), (1, 1, 4200, 4, 2, 1)])
 def test_state_space_recurrence_alone_whole_and_in_portions(heads, groups, vdim, n, taps, parts, dtype):
     """The mixer on hand-made steps: two requests side by side, cut into portions of unequal lengths (one token, two,
     fewer than the convolution has taps, many), each carried by its state slot; against the plain recurrence.  Portions
