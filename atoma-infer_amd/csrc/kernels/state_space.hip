@@ -11,8 +11,8 @@
 //   ssd_scan         per (request, head, 16 columns of S): the recurrence over the entry's tokens in order, S read from
 //                    the request's state slot before and written back after.  A column of S lives in the registers of
 //                    16 neighbouring lanes (n / 16 rows each, rounded up); the tokens' inputs pass LDS in blocks;
-//   ssd_chunk        the same recurrence for entries of many tokens (prompts and their portions), 64 tokens at a time on
-//                    the matrix cores in float32 (v_mfma_f32_16x16x4_f32), see below;
+//   ssd_scores,      the same recurrence for entries of many tokens (prompts and their portions), 64 tokens at a time on
+//   ssd_chunk        the matrix cores in float32 (v_mfma_f32_16x16x4_f32), see below;
 //   ssd_out          per token and norm group: y * silu(z), divided by the root mean square of its group, times the
 //                    weight, in the activation dtype.
 // The order of every sum depends on the sizes alone, so a token's result does not depend on how the request was cut
@@ -164,9 +164,11 @@ ssd_scan_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, con
 // The recurrence 64 tokens at a time.  With c_t the sum of the log decays of the chunk's tokens up to t (inclusive),
 //   y_t = sum_{s <= t} exp(c_t - c_s) dt_s (C_t . B_s) x_s  +  exp(c_t) S_0^T C_t  +  D x_t,
 //   S_64 = exp(c_63) S_0 + sum_s exp(c_63 - c_s) dt_s B_s x_s^T,
-// every exponent at most zero.  A workgroup owns (entry, head, 16 columns of S) and walks the entry's chunks in order;
-// per chunk its four waves make M[t][s] = (C_t . B_s) exp(c_t - c_s) dt_s for s <= t (ten tiles of 16 x 16 shared out
-// among them, into LDS), then each takes 16 tokens of y = M X + diag(exp(c)) C S, then each its share of the rows of S.
+// every exponent at most zero.  The products C_t . B_s are the same for all heads of a group and all columns of S: a
+// first kernel (ssd_scores) makes them once per (chunk, group).  Then a workgroup owns (entry, head, 16 columns of S)
+// and walks the entry's chunks in order; per chunk its four waves make M[t][s] = (C_t . B_s) exp(c_t - c_s) dt_s for
+// s <= t (ten tiles of 16 x 16 shared out among them, into LDS), then each takes 16 tokens of
+// y = M X + diag(exp(c)) C S, then each its share of the rows of S.
 // All products are float32 MFMAs of 16 x 16 x 4 (result D[4 (l / 16) + i][l % 16] in lane l).  The sum over k of a
 // block of 16 is taken in the order that lets a lane fetch its four values with one 16-byte load from LDS: in the
 // block's MFMA j, lane l gives A[l % 16][4 (l / 16) + j] and B[4 (l / 16) + j][l % 16]; tiles whose k runs along their
@@ -182,12 +184,14 @@ __host__ __device__ constexpr int chunk_lds_floats(int nb) {
 
 __device__ __forceinline__ f32x4 lds4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
 
-template <int NB>      // blocks of 16 rows of S (the state size rounded up)
+// VEC: B and C rows are fetched and put into LDS 16 bytes at a time (state size, channel counts and the first column
+// of the group's B all multiples of 4)
+template <int NB, bool VEC>      // NB: blocks of 16 rows of S (the state size rounded up)
 __global__ void __launch_bounds__(256)
 ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, const float* __restrict__ a_log,
                  const float* __restrict__ d_skip, SsdShape sh, const int32_t* __restrict__ q_start,
                  const int32_t* __restrict__ state_slots, float* __restrict__ state, size_t state_stride,
-                 float* __restrict__ y, int at_least) {
+                 float* __restrict__ y, int at_least, const float* __restrict__ scores, int max_chunks) {
   constexpr int NP = 16 * NB, LDN = NP + 4;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float* Bs = lds;                         // [kChunk][LDN]   B of the chunk's tokens
@@ -217,16 +221,38 @@ ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, co
   // A chunk's B, C, x and dt are asked for while the chunk before is worked on, and wait in registers meanwhile.
   constexpr int PER = kChunk * NP / 256;        // elements of a [64][NP] tile a thread moves
   float rb[PER], rc[PER], rx[4], rdt = 0.f;
+  f32x4 mt[3];       // the wave's tiles of C . B of the chunk, as the scores kernel left them
   auto fetch = [&](int t0) {
     const int nt = min(kChunk, count - t0);
     const size_t tok0 = (size_t)(first + t0);
+    const float* sc = scores + (((size_t)e * max_chunks + t0 / kChunk) * sh.groups + g) * (10 * 256);
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int idx = tid + i * 256, tt = idx / NP, n = idx % NP;
-      const bool in = tt < nt && n < sh.n;
-      const size_t base = (tok0 + tt) * channels + inner + (size_t)g * sh.n + n;
-      rb[i] = in ? xbc[base] : 0.f;
-      rc[i] = in ? xbc[base + gn] : 0.f;
+    for (int m = 0; m < 3; ++m)      // tile wave + 4 m is the wave's m-th
+      if (wave + 4 * m < 10) mt[m] = *reinterpret_cast<const f32x4*>(sc + ((wave + 4 * m) * 64 + lane) * 4);
+    if constexpr (VEC) {
+#pragma unroll
+      for (int i = 0; i < PER / 4; ++i) {
+        const int idx = tid + i * 256, tt = idx / (NP / 4), n = (idx % (NP / 4)) * 4;
+        const bool in = tt < nt && n < sh.n;
+        const size_t base = (tok0 + tt) * channels + inner + (size_t)g * sh.n + n;
+        const f32x4 zero = f32x4{0.f, 0.f, 0.f, 0.f};
+        const f32x4 b4 = in ? *reinterpret_cast<const f32x4*>(xbc + base) : zero;
+        const f32x4 c4 = in ? *reinterpret_cast<const f32x4*>(xbc + base + gn) : zero;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          rb[4 * i + q] = b4[q];
+          rc[4 * i + q] = c4[q];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int idx = tid + i * 256, tt = idx / NP, n = idx % NP;
+        const bool in = tt < nt && n < sh.n;
+        const size_t base = (tok0 + tt) * channels + inner + (size_t)g * sh.n + n;
+        rb[i] = in ? xbc[base] : 0.f;
+        rc[i] = in ? xbc[base + gn] : 0.f;
+      }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -240,11 +266,20 @@ ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, co
     const int nt = min(kChunk, count - t0);
     const size_t tok0 = (size_t)(first + t0);
     __syncthreads();       // the chunk before is done with every tile
+    if constexpr (VEC) {
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int idx = tid + i * 256, tt = idx / NP, n = idx % NP;
-      Bs[tt * LDN + n] = rb[i];
-      Cs[tt * LDN + n] = rc[i];
+      for (int i = 0; i < PER / 4; ++i) {
+        const int idx = tid + i * 256, tt = idx / (NP / 4), n = (idx % (NP / 4)) * 4;
+        *reinterpret_cast<f32x4*>(Bs + tt * LDN + n) = f32x4{rb[4 * i], rb[4 * i + 1], rb[4 * i + 2], rb[4 * i + 3]};
+        *reinterpret_cast<f32x4*>(Cs + tt * LDN + n) = f32x4{rc[4 * i], rc[4 * i + 1], rc[4 * i + 2], rc[4 * i + 3]};
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int idx = tid + i * 256, tt = idx / NP, n = idx % NP;
+        Bs[tt * LDN + n] = rb[i];
+        Cs[tt * LDN + n] = rc[i];
+      }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -253,7 +288,6 @@ ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, co
     }
     if (tid < kChunk) dts[tid] = rdt;
     __syncthreads();
-    if (t0 + kChunk < count) fetch(t0 + kChunk);
     if (wave == 0) {
       // inclusive sums of the log decays over the 64 lanes
       float c = -rate * dts[lane];
@@ -267,25 +301,7 @@ ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, co
       wts[lane] = expf(last - c) * dts[lane];
       ect[lane] = expf(c);
     }
-    // M: the ten tiles on and below the diagonal, dealt to the waves in turn (the products need no decay yet)
-    // (tile j is the wave's (j / 4)-th; the loops are unrolled, so the tiles wait in registers named at compile time)
-    f32x4 mt[3];
-#pragma unroll
-    for (int j = 0; j < 10; ++j) {
-      const int tb = j >= 6 ? 3 : j >= 3 ? 2 : j >= 1 ? 1 : 0, sb = j - tb * (tb + 1) / 2;
-      if ((j & 3) == wave) {
-        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-        const float* cp = Cs + (tb * 16 + r16) * LDN + 4 * kg;
-        const float* bp = Bs + (sb * 16 + r16) * LDN + 4 * kg;
-#pragma unroll
-        for (int k = 0; k < NP; k += 16) {
-          const f32x4 a4 = lds4(cp + k), b4 = lds4(bp + k);
-#pragma unroll
-          for (int q = 0; q < 4; ++q) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[q], b4[q], acc, 0, 0, 0);
-        }
-        mt[j >> 2] = acc;
-      }
-    }
+    // (the chunk after this one is fetched further down, when this chunk's tiles of scores have been used)
     __syncthreads();       // the sums of the log decays are there
 #pragma unroll
     for (int j = 0; j < 10; ++j) {
@@ -301,6 +317,7 @@ ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, co
         }
       }
     }
+    if (t0 + kChunk < count) fetch(t0 + kChunk);
     __syncthreads();
     // y of the wave's 16 tokens
     if (wave * 16 < nt) {
@@ -356,6 +373,50 @@ ssd_chunk_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, co
   for (int idx = tid; idx < NP * 16; idx += 256) {
     const int v = idx / NP, n = idx % NP;
     if (v < vlive && n < sh.n) s_ptr[(size_t)v * sh.n + n] = St[v * LDN + n];
+  }
+}
+
+// C_t . B_s of every chunk of 64 tokens, once per group of heads: the ten 16 x 16 tiles on and below the diagonal, each
+// as its 64 lanes' four numbers (lane l: rows 4 (l / 16) .. + 3, column l % 16 of the tile), [entry][chunk][group][10][64][4].
+template <int NB>
+__global__ void __launch_bounds__(256)
+ssd_scores_kernel(const float* __restrict__ xbc, SsdShape sh, const int32_t* __restrict__ q_start, int at_least,
+                  float* __restrict__ scores, int max_chunks) {
+  constexpr int NP = 16 * NB, LDN = NP + 4;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* Bs = lds;
+  float* Cs = Bs + kChunk * LDN;
+  const int e = blockIdx.z, g = blockIdx.y, t0 = blockIdx.x * kChunk;
+  const int first = q_start[e], count = q_start[e + 1] - first;
+  if (count < at_least || t0 >= count) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int inner = sh.heads * sh.vdim, gn = sh.groups * sh.n, channels = inner + 2 * gn;
+  const int nt = min(kChunk, count - t0);
+  for (int idx = tid; idx < kChunk * NP; idx += 256) {
+    const int tt = idx / NP, n = idx % NP;
+    const bool in = tt < nt && n < sh.n;
+    const size_t base = ((size_t)(first + t0) + tt) * channels + inner + (size_t)g * sh.n + n;
+    Bs[tt * LDN + n] = in ? xbc[base] : 0.f;
+    Cs[tt * LDN + n] = in ? xbc[base + gn] : 0.f;
+  }
+  __syncthreads();
+  float* out = scores + (((size_t)e * max_chunks + blockIdx.x) * sh.groups + g) * (10 * 256);
+#pragma unroll
+  for (int j = 0; j < 10; ++j) {
+    const int tb = j >= 6 ? 3 : j >= 3 ? 2 : j >= 1 ? 1 : 0, sb = j - tb * (tb + 1) / 2;
+    if ((j & 3) == wave) {
+      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+      const float* cp = Cs + (tb * 16 + r16) * LDN + 4 * kg;
+      const float* bp = Bs + (sb * 16 + r16) * LDN + 4 * kg;
+#pragma unroll
+      for (int k = 0; k < NP; k += 16) {
+        const f32x4 a4 = lds4(cp + k), b4 = lds4(bp + k);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[q], b4[q], acc, 0, 0, 0);
+      }
+      *reinterpret_cast<f32x4*>(out + (j * 64 + lane) * 4) = acc;
+    }
   }
 }
 
@@ -470,43 +531,69 @@ extern "C" int atoma_ssd_scan(const float* xbc, const float* dt, const float* de
 // The largest state size the chunk kernel takes (its tiles of B and C must fit the CU's LDS beside the rest).
 extern "C" int atoma_ssd_chunk_max_state() { return 128; }
 
-template <int NB>
+template <int NB, bool VEC>
 static int launch_chunk(dim3 grid, hipStream_t stream, const float* xbc, const float* dt, const float* a_log,
                         const float* d_skip, const SsdShape& sh, const int32_t* q_start, const int32_t* state_slots,
-                        float* state, size_t state_stride, float* y, int at_least) {
+                        float* state, size_t state_stride, float* y, int at_least, float* scores, int max_chunks) {
   const size_t bytes = (size_t)chunk_lds_floats(NB) * sizeof(float);
+  const size_t sbytes = (size_t)2 * kChunk * (16 * NB + 4) * sizeof(float);
   static bool asked = false;      // (per instantiation) more than the default 64 KB of LDS
-  if (!asked && bytes > 64 * 1024) {
-    hipError_t err = hipFuncSetAttribute((const void*)ssd_chunk_kernel<NB>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)bytes);
-    if (err != hipSuccess) return (int)err;
+  if (!asked) {
+    if (bytes > 64 * 1024) {
+      hipError_t err = hipFuncSetAttribute((const void*)ssd_chunk_kernel<NB, VEC>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+      if (err != hipSuccess) return (int)err;
+    }
+    if (sbytes > 64 * 1024) {
+      hipError_t err = hipFuncSetAttribute((const void*)ssd_scores_kernel<NB>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)sbytes);
+      if (err != hipSuccess) return (int)err;
+    }
     asked = true;
   }
-  hipLaunchKernelGGL((ssd_chunk_kernel<NB>), grid, dim3(256), bytes, stream, xbc, dt, a_log, d_skip, sh, q_start,
-                     state_slots, state, state_stride, y, at_least);
+  hipLaunchKernelGGL((ssd_scores_kernel<NB>), dim3(max_chunks, sh.groups, grid.z), dim3(256), sbytes, stream, xbc, sh,
+                     q_start, at_least, scores, max_chunks);
+  hipLaunchKernelGGL((ssd_chunk_kernel<NB, VEC>), grid, dim3(256), bytes, stream, xbc, dt, a_log, d_skip, sh, q_start,
+                     state_slots, state, state_stride, y, at_least, scores, max_chunks);
   return 0;
 }
 
-// entries of at least `at_least` tokens; the others are left to atoma_ssd_scan(below = at_least)
+// Floats of scratch that atoma_ssd_chunk needs for entries of up to `max_chunks` chunks of 64 tokens.
+extern "C" size_t atoma_ssd_chunk_scratch_floats(int n_entries, int max_chunks, int groups) {
+  return (size_t)n_entries * max_chunks * groups * 10 * 256;
+}
+
+// entries of at least `at_least` tokens; the others are left to atoma_ssd_scan(below = at_least).  `max_chunks`: chunks
+// of 64 tokens of the longest entry; `scores`: scratch of atoma_ssd_chunk_scratch_floats floats.
 extern "C" int atoma_ssd_chunk(const float* xbc, const float* dt, const float* a_log, const float* d_skip, int heads,
                                int groups, int vdim, int n, int taps, const int32_t* q_start,
                                const int32_t* state_slots, float* state, size_t state_stride, float* y,
-                               int n_entries, int at_least, hipStream_t stream) {
+                               int n_entries, int at_least, float* scores, int max_chunks, hipStream_t stream) {
   if (n_entries <= 0) return 0;
   SsdShape sh{heads, groups, vdim, n, taps, 1, 0, 0, 0};
-  if (!shape_ok(sh) || n > 128 || n_entries > 65535 || heads > 65535 || at_least < 1) return ATOMA_ERR_SHAPE;
+  if (!shape_ok(sh) || n > 128 || n_entries > 65535 || heads > 65535 || groups > 65535 || at_least < 1 ||
+      max_chunks < 1 || scores == nullptr)
+    return ATOMA_ERR_SHAPE;
   dim3 grid((vdim + 15) / 16, heads, n_entries);
   int rc;
+  // (a state size that is a multiple of 4 is then also a whole number of 16-byte pieces of its NB blocks' row)
+  const bool vec = n % 4 == 0 && (heads * vdim) % 4 == 0 && ((uintptr_t)xbc & 15) == 0;
+#define ATOMA_CHUNK(NB_)                                                                                            \
+  rc = vec ? launch_chunk<NB_, true>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state,        \
+                                     state_stride, y, at_least, scores, max_chunks)                               \
+           : launch_chunk<NB_, false>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state,       \
+                                      state_stride, y, at_least, scores, max_chunks)
   switch ((n + 15) / 16) {
-    case 1: rc = launch_chunk<1>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
-    case 2: rc = launch_chunk<2>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
-    case 3: rc = launch_chunk<3>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
-    case 4: rc = launch_chunk<4>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
-    case 5: rc = launch_chunk<5>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
-    case 6: rc = launch_chunk<6>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
-    case 7: rc = launch_chunk<7>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
-    default: rc = launch_chunk<8>(grid, stream, xbc, dt, a_log, d_skip, sh, q_start, state_slots, state, state_stride, y, at_least); break;
+    case 1: ATOMA_CHUNK(1); break;
+    case 2: ATOMA_CHUNK(2); break;
+    case 3: ATOMA_CHUNK(3); break;
+    case 4: ATOMA_CHUNK(4); break;
+    case 5: ATOMA_CHUNK(5); break;
+    case 6: ATOMA_CHUNK(6); break;
+    case 7: ATOMA_CHUNK(7); break;
+    default: ATOMA_CHUNK(8); break;
   }
+#undef ATOMA_CHUNK
   if (rc != 0) return rc;
   ATOMA_LAUNCH_CHECK();
   return 0;

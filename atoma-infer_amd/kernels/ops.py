@@ -567,9 +567,13 @@ def ssd_scan(xbc: torch.Tensor, dt: torch.Tensor, decay: torch.Tensor, a_log: to
     below = 1 << 30
     if longest >= SSD_CHUNK_MIN_TOKENS:
         below = SSD_CHUNK_MIN_TOKENS
+        max_chunks = -(-longest // 64)
+        lib.atoma_ssd_chunk_scratch_floats.restype = ctypes.c_size_t
+        scores = torch.empty((lib.atoma_ssd_chunk_scratch_floats(s, max_chunks, groups),), dtype=torch.float32,
+                             device=xbc.device)
         _check(lib.atoma_ssd_chunk(
             _p(xbc), _p(dt), _p(a_log), _p(d_skip), heads, groups, vdim, n, taps, _p(q_start), _p(state_slots), _p(state),
-            ctypes.c_size_t(state.stride(0)), _p(y), s, below, _stream()), "ssd_chunk")
+            ctypes.c_size_t(state.stride(0)), _p(y), s, below, _p(scores), max_chunks, _stream()), "ssd_chunk")
     if shortest < below:
         _check(lib.atoma_ssd_scan(
             _p(xbc), _p(dt), _p(decay), _p(d_skip), heads, groups, vdim, n, taps, _p(q_start), _p(state_slots), _p(state),
