@@ -86,55 +86,65 @@ head_linear_kernel(const TA* __restrict__ x, int ldx, const TW* __restrict__ w, 
 }
 
 // The same on the matrix cores for bfloat16 operands (v_mfma_f32_16x16x32_bf16, float32 sums): a workgroup takes 64
-// tokens x 64 outputs of one head, a wave 16 of the outputs against all 64 tokens; both operands' fragments come
-// straight from memory (K is a head's width: a few steps).  K a multiple of 8; a last step shorter than 32 columns is
-// filled with zeros.  The MFMA's result holds, per lane, token (lane % 16) and outputs (lane / 16) * 4 .. + 3.
+// tokens x 16 NS outputs of one head, a wave 16 of the tokens against all of those outputs, so that a token's row is
+// fetched by one wave only and what the waves fetch in common is the head's weight, which is small and stays in the
+// caches.  Both operands' fragments come straight from memory (K is a head's width: a few steps), four steps of 32
+// columns asked for at a time.  K a multiple of 8; a last step shorter than 32 columns is filled with zeros.  The
+// MFMA's result holds, per lane, token (lane % 16) and outputs (lane / 16) * 4 .. + 3.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
-template <typename TO>
+template <typename TO, int NS>
 __global__ void __launch_bounds__(256)
 head_linear_mfma_kernel(const uint16_t* __restrict__ x, int ldx, const uint16_t* __restrict__ w, TO* __restrict__ out,
                         int ldo, const float* __restrict__ gate, int T, int H, int K, int N) {
-  const int h = blockIdx.z, n0 = blockIdx.x * 64, t0 = blockIdx.y * 64;
+  const int h = blockIdx.z, n0 = blockIdx.x * (16 * NS);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
-  const int msub = min(4, (T - t0 + 15) >> 4);
-  int n = n0 + wave * 16 + r16;
-  if (n > N - 1) n = N - 1;                                  // clamped rows are computed and never stored
-  const uint16_t* wp = w + ((size_t)h * N + n) * K + kg * 8;
-  const uint16_t* xp[4];
+  const int tb = blockIdx.y * 64 + wave * 16;              // the wave's 16 tokens
+  if (tb >= T) return;
+  int t = tb + r16;
+  if (t > T - 1) t = T - 1;                                // clamped rows are computed and never stored
+  const uint16_t* xp = x + (size_t)t * ldx + (size_t)h * K + kg * 8;
+  const uint16_t* wp[NS];
 #pragma unroll
-  for (int m = 0; m < 4; ++m) {
-    int t = t0 + m * 16 + r16;
-    if (t > T - 1) t = T - 1;
-    xp[m] = x + (size_t)t * ldx + (size_t)h * K + kg * 8;
+  for (int s = 0; s < NS; ++s) {
+    int n = n0 + s * 16 + r16;
+    if (n > N - 1) n = N - 1;
+    wp[s] = w + ((size_t)h * N + n) * K + kg * 8;
   }
-  f32x4 acc[4];
+  f32x4 acc[NS];
 #pragma unroll
-  for (int m = 0; m < 4; ++m) acc[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < NS; ++s) acc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    const bool in = k0 + kg * 8 < K;
-    const bf16x8 wf = in ? *reinterpret_cast<const bf16x8*>(wp + k0) : zero;
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    bf16x8 xf[2], wf[2][NS];
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      if (m < msub) {
-        const bf16x8 xf = in ? *reinterpret_cast<const bf16x8*>(xp[m] + k0) : zero;
-        acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf, acc[m], 0, 0, 0);
+    for (int st = 0; st < 2; ++st) {
+      const int k = k0 + 32 * st;
+      const bool in = k + kg * 8 < K;
+      xf[st] = in ? *reinterpret_cast<const bf16x8*>(xp + k) : zero;
+#pragma unroll
+      for (int s = 0; s < NS; ++s) wf[st][s] = in ? *reinterpret_cast<const bf16x8*>(wp[s] + k) : zero;
+    }
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      if (k0 + 32 * st < K) {
+#pragma unroll
+        for (int s = 0; s < NS; ++s) acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[st][s], xf[st], acc[s], 0, 0, 0);
       }
     }
   }
-  const int nb = n0 + wave * 16 + kg * 4;
+  t = tb + r16;
+  if (t >= T) return;
+  const float g = gate ? gate[(size_t)t * H + h] : 1.0f;
 #pragma unroll
-  for (int m = 0; m < 4; ++m) {
-    const int t = t0 + m * 16 + r16;
-    if (m >= msub || t >= T) continue;
-    const float s = gate ? gate[(size_t)t * H + h] : 1.0f;
+  for (int s = 0; s < NS; ++s) {
+    const int nb = n0 + s * 16 + kg * 4;
     TO* dst = out + (size_t)t * ldo + (size_t)h * N + nb;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (nb + i < N) dst[i] = from_f32<TO>(acc[m][i] * s);
+      if (nb + i < N) dst[i] = from_f32<TO>(acc[s][i] * g);
   }
 }
 
@@ -164,15 +174,21 @@ extern "C" int atoma_head_linear(const void* x, int x_dtype, int ldx, const void
   if (H <= 0 || K <= 0 || N <= 0 || ldx < H * K || ldo < H * N || H > 65535 || (T + 15) / 16 > 65535) return ATOMA_ERR_SHAPE;
   if (x_dtype == kBF16 && w_dtype == kBF16 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x & 15) == 0 &&
       ((uintptr_t)w & 15) == 0 && (T + 63) / 64 <= 65535) {
-    dim3 mgrid((N + 63) / 64, (T + 63) / 64, H);
-    if (out_dtype == kBF16)
-      hipLaunchKernelGGL((head_linear_mfma_kernel<bf16_t>), mgrid, dim3(256), 0, stream, (const uint16_t*)x, ldx,
-                         (const uint16_t*)w, (bf16_t*)out, ldo, gate, T, H, K, N);
-    else if (out_dtype == kF32)
-      hipLaunchKernelGGL((head_linear_mfma_kernel<float>), mgrid, dim3(256), 0, stream, (const uint16_t*)x, ldx,
-                         (const uint16_t*)w, (float*)out, ldo, gate, T, H, K, N);
-    else
+    const bool wide = N > 64;                  // eight blocks of 16 outputs a wave, else four
+    dim3 mgrid((N + (wide ? 127 : 63)) / (wide ? 128 : 64), (T + 63) / 64, H);
+#define ATOMA_HLM(TO, NS)                                                                                          \
+  hipLaunchKernelGGL((head_linear_mfma_kernel<TO, NS>), mgrid, dim3(256), 0, stream, (const uint16_t*)x, ldx,      \
+                     (const uint16_t*)w, (TO*)out, ldo, gate, T, H, K, N)
+    if (out_dtype == kBF16) {
+      if (wide) ATOMA_HLM(bf16_t, 8);
+      else ATOMA_HLM(bf16_t, 4);
+    } else if (out_dtype == kF32) {
+      if (wide) ATOMA_HLM(float, 8);
+      else ATOMA_HLM(float, 4);
+    } else {
       return ATOMA_ERR_DTYPE;
+    }
+#undef ATOMA_HLM
     ATOMA_LAUNCH_CHECK();
     return 0;
   }
