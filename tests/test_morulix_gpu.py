@@ -306,6 +306,26 @@ def test_a_dominant_key_just_inside_and_just_outside_the_window(dtype, edge):
     assert _rel(want[0][p + window - 1], want[0][p + window]) > 0.3
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [300, None])
+def test_a_far_key_under_a_long_window_and_behind_it(dtype, window):
+    """A dominant key hundreds of positions back, at a page's last slot: under a window of 300 keys the rows up to 299
+    positions later are made of its value and the rows behind are not; without a window every later row is.  Rows in a
+    long portion, in portions of two tokens and decoded alone stand on both sides of the edge."""
+    p = 31
+    # (a few columns rotated: the others carry the key's weight over any distance)
+    m = attention(dim=64, heads=4, kv_heads=2, vdim=32, scale=0.6, window=window, rot_dims=8, base=200.0)
+    part, plain = _window_part(m, dtype)
+    edge = p + 300                      # the first position that no longer sees the key under the window
+    cuts = [[(0, 200), (1, 5)], [(0, edge - 200 - 3)], [(0, 2)], [(0, 1)], [(0, 1)], [(0, 2)], [(0, 1)], [(0, 40), (1, 1)]] + \
+        [[(0, 1)]] * 6
+    got, want = _paged_case(part, plain, dtype, cuts, 16, seed=9, boost=(0, p))
+    rows = slice(edge - 4, edge + 4)
+    assert _rel(got[0][rows], want[0][rows]) < PART_TOL[dtype] and _rel(got[0], want[0]) < PART_TOL[dtype]
+    far = _rel(want[0][edge - 1], want[0][edge])
+    assert far > 0.3 if window else far < 0.3        # (the plain rows say whether there is an edge to see)
+
+
 def _latent_part(m, dtype, seed=7, width=64, sink_value=None):
     from atoma_infer_amd.parts import LatentAttention
     part = LatentAttention(width, m["heads"], m["dim"], m["vdim"], m["kv_rank"], m["scale"], 1e-5)
