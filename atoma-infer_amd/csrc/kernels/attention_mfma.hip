@@ -662,7 +662,9 @@ constexpr size_t kLdsBytes = 160 * 1024;
 constexpr size_t kMerge2Bytes = (DTILES * 16 + 2) * 64 * 4 * sizeof(float);
 constexpr size_t kMerge4Bytes = (DTILES * 16 + 2) * 64 * 6 * sizeof(float);      // two tasks, three waves each
 constexpr size_t kMerge8Bytes = (DTILES * 16 + 2) * 64 * 7 * sizeof(float);
-constexpr bool kSplit2Fits = kMerge2Bytes <= kLdsBytes;
+// (heads beyond 192 columns: a wave's output alone is more than a hundred registers a lane, and with the eight waves of
+// a split workgroup a lane may have 256; such heads keep one wave a task and four waves a workgroup)
+constexpr bool kSplit2Fits = kMerge2Bytes <= kLdsBytes && HD <= 192;
 constexpr bool kSplit4Fits = kMerge4Bytes <= kLdsBytes;
 constexpr bool kSplit8Fits = kMerge8Bytes <= kLdsBytes;
 // two pieces of rows a wave: where the accumulators of both fit the registers of eight waves a workgroup, and the

@@ -66,7 +66,8 @@ def max_waves_for(hd: int) -> int:
     per_lane = -(-hd // 32) * 16 + 2
     if per_lane * 64 * 7 * 4 <= 160 * 1024:
         return 8
-    return 2 if per_lane * 64 * 4 * 4 <= 160 * 1024 else 1
+    # (beyond 192 columns a wave's output alone fills the registers that a lane of an eight-wave workgroup may have)
+    return 2 if per_lane * 64 * 4 * 4 <= 160 * 1024 and hd <= 192 else 1
 
 
 TWO_PIECES_MIN_KEYS = 16384     # keys from which on a wave of a prompt step works on two pieces of rows

@@ -186,9 +186,10 @@ def test_whole_ranges_for_many_decoding_requests(seed):
     # wide heads with many tasks: two waves a chunk and the merging kernel, as where fewer than four waves may share
     assert A.chunk_for(8, 32768, 8, whole_ok=True, head_size=128) == (512, 2)
     assert A.chunk_for(12, 32768, 8, whole_ok=False, head_size=64)[1] <= 2
-    # the merge of the waves' shares must fit the 160 KB of LDS of a CU: eight waves up to heads of 160, two beyond
+    # the merge of the waves' shares must fit the 160 KB of LDS of a CU: eight waves up to heads of 160, two beyond; and
+    # beyond 192 columns a wave's output alone fills the registers of a lane in an eight-wave workgroup: one wave a task
     assert A.max_waves_for(64) == 8 and A.max_waves_for(128) == 8 and A.max_waves_for(160) == 8
-    assert A.max_waves_for(176) == 2 and A.max_waves_for(256) == 2
+    assert A.max_waves_for(176) == 2 and A.max_waves_for(192) == 2 and A.max_waves_for(208) == 1 and A.max_waves_for(256) == 1
 
 
 @pytest.mark.parametrize("seed", range(20))
