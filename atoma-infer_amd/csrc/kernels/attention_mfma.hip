@@ -720,7 +720,10 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
                        window, (const uint16_t*)kcache, (const uint16_t*)vcache, (uint16_t*)out, out_stride,       \
                        part_o, part_lse, scale, counters, sinks);                                                  \
   } while (0)
-  if (ksplit == 1) ATOMA_ATTN(4, 1, 0);
+  // (wide heads keep one wave a task, see kSplit2Fits: with few tasks, as in a decode step over one shared key/value
+  // head, a workgroup of four of them would leave most CUs without work, so each task gets a workgroup of its own)
+  if (ksplit == 1 && HD > 192 && (size_t)n_tasks * nkv <= 1024) ATOMA_ATTN(1, 1, 0);
+  else if (ksplit == 1) ATOMA_ATTN(4, 1, 0);
   else if (ksplit == 2 && row_tiles == 2) ATOMA_ATTN(4, 2, 2 * kMerge2Bytes, (kTwoPieces ? 2 : 1));
   else if (ksplit == 2 && kSplit2Fits) ATOMA_ATTN(4, (kSplit2Fits ? 2 : 1), kMerge2Bytes);
   else if (ksplit == 4 && kSplit4Fits) ATOMA_ATTN(2, (kSplit4Fits ? 4 : 1), kMerge4Bytes);
