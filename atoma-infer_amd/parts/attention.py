@@ -360,8 +360,8 @@ class LatentAttention(PagedAttention):
     def device_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_uk, self.w_uv, self.w_o))
 
-    accepts_begun = False
-    takes_sink = False
+    accepts_begun = True
+    takes_sink = True
 
     def forward(self, x, ctx, cache, sink=None):
         if not cache.writable:
@@ -373,10 +373,10 @@ class LatentAttention(PagedAttention):
                                      self.c_norm, self.norm_eps, cache.k, cache.v, cache.slot_mapping,
                                      cache.page_size, x.dtype)
         ql = ops.head_linear(q, self.w_uk, x.dtype)                      # the queries in the latent's columns
-        mixed = torch.empty((t, self.nh * self.hd), dtype=x.dtype, device=x.device)
+        mixed = torch.empty((t, self.nh * self.hd), dtype=x.dtype, device=proj.device)
         self.attend(ql, cache.k, cache.v, mixed, ctx, cache)
         out = ops.head_linear(mixed, self.w_uv, x.dtype, gate)           # the heads' values, gated
-        return linear_delta(out, self.w_o, None, self.w_o_tiled)
+        return linear_delta(out, self.w_o, sink, self.w_o_tiled)
 
 
 register_mixer("latent_attention", LatentAttention)

@@ -15,8 +15,13 @@ from __future__ import annotations
 
 from typing import Dict, Optional
 
+import torch
+
+from ..kernels import ops
 from .base import Begun, Block, FeedForward, Mixer, Norm, WeightSpec, register_block
 from .linear import Normed, ResidualSink
+
+BEGUN_ROWS = 16      # rows of a step up to which products begin and finish norms (kernels.gemm_bf16.BEGUN_MAX_M)
 
 
 class PreNormBlock(Block):
@@ -157,13 +162,39 @@ class SideBySideBlock(Block):
     def device_bytes(self) -> int:
         return sum(part.device_bytes() for _, part in self._children())
 
-    def forward(self, resid, delta, ctx, cache):
+    fuses_next_norm = True
+
+    def entry_norm(self):
+        return self.norm1
+
+    def forward(self, resid, delta, ctx, cache, next_norm=None):
         from .base import WeightedSum
-        x = self.norm1.add_norm(resid, delta)
-        a = self.mixer.forward(x, ctx, cache)
+        if isinstance(delta, (Normed, Begun)):
+            # the block before has added its outputs to the stream and begun or finished this block's norm
+            if delta.norm is not self.norm1:
+                raise RuntimeError("a begun or finished norm reached another norm than the one it was made for")
+            x = delta.data if isinstance(delta, Normed) else delta
+        else:
+            x = self.norm1.add_norm(resid, delta)
+        few = isinstance(x, Begun) or (x.dtype is torch.bfloat16 and x.shape[0] <= BEGUN_ROWS)
+
+        def reads(part):
+            return x if not isinstance(x, Begun) or part.accepts_begun else x.tensor()
+
         if self.feed_forward is None:
-            return a
-        return WeightedSum([(a, 1.0), (self.feed_forward.forward(x, ctx), 1.0)])
+            if self.mixer.takes_sink and few and next_norm is not None:
+                return self.mixer.forward(reads(self.mixer), ctx, cache, sink=ResidualSink(resid, next_norm))
+            return self.mixer.forward(reads(self.mixer), ctx, cache)
+        # Steps of few rows: both sublayers' last products add themselves to the stream's rows (the mixer's first, so
+        # that the feed-forward's, which also begins the next norm, sees the rows complete), and no kernel of its own
+        # sums them.  What the mixer's product begins of a norm is dropped: its rows lacked the feed-forward's share.
+        if few and next_norm is not None and self.mixer.takes_sink and self.feed_forward.takes_sink:
+            a = self.mixer.forward(reads(self.mixer), ctx, cache, sink=ResidualSink(resid, next_norm))
+            if not isinstance(a, (Begun, Normed)):      # the product could not: its delta joins the stream here
+                ops.add_normed(resid, a.terms if isinstance(a, WeightedSum) else [(a, 1.0)], None, 0.0)
+            return self.feed_forward.forward(reads(self.feed_forward), ctx, sink=ResidualSink(resid, next_norm))
+        a = self.mixer.forward(reads(self.mixer), ctx, cache)
+        return WeightedSum([(a, 1.0), (self.feed_forward.forward(reads(self.feed_forward), ctx), 1.0)])
 
 
 register_block("pre_norm", PreNormBlock)

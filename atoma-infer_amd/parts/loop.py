@@ -17,8 +17,8 @@ from typing import Dict, Optional
 import torch
 
 from ..kernels import ops
-from .base import Block, Mixer, WeightedSum, WeightSpec, register_block, register_mixer
-from .linear import linear
+from .base import Begun, Block, Mixer, WeightedSum, WeightSpec, register_block, register_mixer
+from .linear import Normed, linear
 
 
 class NoMixer(Mixer):
@@ -63,7 +63,9 @@ class LoopEntry(Block):
     def forward(self, resid, delta, ctx, cache, embedded=None, turn=0):
         if embedded is None or not 0 <= turn < self.times:
             raise RuntimeError("a loop entry needs the embedding's rows and a pass number below its number of passes")
-        if delta is not None:           # what the block before left pending joins the stream first
+        if isinstance(delta, (Begun, Normed)):
+            pass                        # the block before has added its outputs to the stream already
+        elif delta is not None:         # what the block before left pending joins the stream first
             terms = delta.terms if isinstance(delta, WeightedSum) else [(delta, 1.0)]
             ops.add_normed(resid, terms, None, 0.0)
         pair = ops.pack_pair(resid, embedded, self.act_dtype if self.w_in.dtype is torch.bfloat16 else torch.float32)

@@ -62,7 +62,7 @@ class RMSNorm(Norm):
     # the norm begun by its neighbours (bfloat16 steps of at most 16 rows): see kernels/gemm_bf16.py; with many rows
     # the library adds its product to the residual rows itself, and the norm reads them once
     def add_product(self, resid, x, w, tiled=None):
-        if self.act_dtype is not torch.bfloat16 or w.dtype is not torch.bfloat16 or self.weight.dtype is not torch.bfloat16:
+        if self.act_dtype is not torch.bfloat16 or w.dtype is not torch.bfloat16:
             return None
         from ..kernels import gemm_bf16
         from .linear import Normed, as_tensor
@@ -75,8 +75,7 @@ class RMSNorm(Norm):
         return None
 
     def embed(self, table, tokens):
-        if self.act_dtype is not torch.bfloat16 or tokens.numel() > 16 or table.shape[1] != self.width \
-                or self.weight.dtype is not torch.bfloat16:
+        if self.act_dtype is not torch.bfloat16 or tokens.numel() > 16 or table.shape[1] != self.width:
             return None
         resid, u, ss = ops.embed_begin_norm(tokens, table, self.weight)
         return resid, Begun(u, ss, self.eps, self.width, self)

@@ -198,7 +198,10 @@ class StateSpaceDuality(Mixer):
     def device_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_o))
 
-    def forward(self, x, ctx, cache):
+    accepts_begun = True
+    takes_sink = True
+
+    def forward(self, x, ctx, cache, sink=None):
         state = cache.state
         dims = (self.heads, self.groups, self.vdim, self.n, self.taps)
         proj = linear(x, self.w_in, torch.float32)
@@ -208,7 +211,7 @@ class StateSpaceDuality(Mixer):
         y = ops.ssd_scan(xbc, dt, decay, self.a_log, self.d_skip, *dims, ctx.q_start, ctx.state_slots, state,
                          counts=ctx.h_counts)
         u = ops.ssd_out(y, proj, self.off_z, self.norm_w, self.norm_eps, self.norm_groups, x.dtype)
-        return linear_delta(u, self.w_o, None, self.w_o_tiled)
+        return linear_delta(u, self.w_o, sink, self.w_o_tiled)
 
 
 register_mixer("gated_delta_rule", GatedDeltaRule)
